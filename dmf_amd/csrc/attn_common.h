@@ -1,0 +1,237 @@
+// Shared device primitives for the gfx950 (MI355X) attention kernels.
+//
+// Register/lane conventions used everywhere (wave64, MFMA 32x32 tiles):
+//   lane = threadIdx.x & 63,  c32 = lane & 31,  g = lane >> 5.
+//   A 32x32 fp32 accumulator tile `acc[16]` of a lane holds
+//       row(i) = (i/4)*8 + 4*g + (i%4),   col = c32.
+//   An MFMA operand "chunk" is one 16-byte vector per lane:
+//     bf16: 8 elements = contraction slots of ONE v_mfma_f32_32x32x16_bf16,
+//     fp32: 4 elements = the operand of FOUR v_mfma_f32_32x32x2_f32.
+//   Both operands of a product always use the same slot->index mapping, so
+//   any consistent permutation of the contraction index is legal; the kernels
+//   exploit that to feed accumulator tiles straight back in as operands.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+namespace dmf {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Exchange between lane and lane^32 (the two halves of a 32x32 tile column).
+__device__ __forceinline__ float xhalf_max(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xhalf_sum(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  f32x2 x = {a, b};
+  bf16x2 y = __builtin_convertvector(x, bf16x2);  // v_cvt_pk_bf16_f32, round-to-nearest-even
+  return __builtin_bit_cast(uint32_t, y);
+}
+
+// Static configuration for element type T (float or __bf16) and head dim D.
+template <typename T, int D>
+struct Cfg {
+  static_assert(D % 8 == 0 && D >= 16 && D <= 128, "head dim must be a multiple of 8 in [16,128]");
+  static constexpr bool BF = sizeof(T) == 2;
+  static constexpr int VEC = 16 / (int)sizeof(T);              // elements per 16-byte vector
+  static constexpr int VPR = D / VEC;                          // valid vectors per row
+  static constexpr int NCHUNK = BF ? (D + 15) / 16 : D / 8;    // operand chunks over the head dim
+  static constexpr int NDT = (D + 31) / 32;                    // 32-wide output tiles over the head dim
+  static constexpr int ROWV0 = (2 * NCHUNK > VPR ? 2 * NCHUNK : VPR);
+  static constexpr int ROWV = ROWV0 + 1 + (ROWV0 & 1);         // LDS row pitch in vectors, odd => conflict-free b128 reads
+  static constexpr int STRIDE = ROWV * VEC;                    // LDS row pitch in elements
+  static constexpr int OROWV = NDT * 32 / VEC + 1;             // epilogue staging pitch (vectors, odd)
+  static constexpr int OSTRIDE = OROWV * VEC;
+  static constexpr int NSUB = BF ? 2 : 1;                      // 32-row sub-tiles per KV tile
+  static constexpr int BKV = 32 * NSUB;
+  static constexpr int TILE_BYTES = BKV * ROWV * 16;
+  static constexpr int PV_STEPS = BF ? 2 : 16;                 // operand steps per 32-row sub-tile in P*V-like products
+};
+
+// acc += A_chunk * B_chunk  (one 16-byte operand chunk per lane each).
+template <typename T>
+__device__ __forceinline__ void mma_chunk(f32x16& acc, const u32x4& a, const u32x4& b) {
+  if constexpr (sizeof(T) == 2) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[e]), __uint_as_float(b[e]), acc, 0, 0, 0);
+  }
+}
+
+// Operand chunk c of row `row` of a row-major LDS tile (contraction along the row).
+template <typename T, int STRIDE>
+__device__ __forceinline__ u32x4 lds_row_chunk(const T* tile, int row, int c, int g) {
+  return *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(tile) + (size_t)row * STRIDE * sizeof(T) + (2 * c + g) * 16);
+}
+
+// "Column" operand for products that contract over the ROWS of a row-major LDS
+// tile (P*V-like): the lane's M index is column col0 + c32 and the contraction
+// slots follow the accumulator row order of the lane (see header comment), so
+// an accumulator tile converted with acc_operand() is the matching B operand.
+//   bf16: step s in {0,1} covers rows r0+16s .. r0+16s+15 (two ds_read_b64_tr_b16).
+//   fp32: step s in 0..15 covers row r0 + (s/4)*8 + 4g + s%4.
+struct ColOperand { u32x4 v; };
+
+template <typename T, int STRIDE>
+__device__ __forceinline__ ColOperand lds_col_operand(const T* tile, int r0, int col0, int s, int lane) {
+  ColOperand r;
+  if constexpr (sizeof(T) == 2) {
+    const int g = lane >> 5, i = lane & 15, half = (lane >> 4) & 1;
+    // 16 lanes cooperatively fetch a 4(row) x 16(col) block; lane i supplies row i/4, cols 4*(i%4)..+3
+    const T* p = tile + (r0 + 16 * s + 4 * g + (i >> 2)) * STRIDE + col0 + 16 * half + 4 * (i & 3);
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * STRIDE));
+    u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+    r.v = u32x4{a[0], a[1], b[0], b[1]};
+  } else {
+    const int g = lane >> 5, c32 = lane & 31;
+    const int row = r0 + (s >> 2) * 8 + 4 * g + (s & 3);
+    r.v = u32x4{__float_as_uint(tile[row * STRIDE + col0 + c32]), 0u, 0u, 0u};
+  }
+  return r;
+}
+
+// Matching B operand built from a lane's accumulator tile (already converted to
+// the probabilities / weights to be contracted).
+template <typename T>
+__device__ __forceinline__ ColOperand acc_operand(const f32x16& e, int s) {
+  ColOperand r;
+  if constexpr (sizeof(T) == 2) {
+    r.v = u32x4{pack_bf16x2(e[8 * s + 0], e[8 * s + 1]), pack_bf16x2(e[8 * s + 2], e[8 * s + 3]),
+                pack_bf16x2(e[8 * s + 4], e[8 * s + 5]), pack_bf16x2(e[8 * s + 6], e[8 * s + 7])};
+  } else {
+    r.v = u32x4{__float_as_uint(e[s]), 0u, 0u, 0u};
+  }
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void mma_col(f32x16& acc, const ColOperand& a, const ColOperand& b) {
+  if constexpr (sizeof(T) == 2) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a.v), __builtin_bit_cast(bf16x8, b.v), acc, 0, 0, 0);
+  } else {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.v[0]), __uint_as_float(b.v[0]), acc, 0, 0, 0);
+  }
+}
+
+// Row index inside a 32-row tile held by accumulator element i of a lane in half g.
+__device__ __forceinline__ int acc_row(int i, int g) { return (i >> 2) * 8 + 4 * g + (i & 3); }
+
+// XCD-aware work-group remap: hardware deals consecutive work-group ids round
+// robin over the 8 XCDs (each with a private L2).  Give every XCD a contiguous
+// range of logical ids so the q-blocks that share one head's K/V hit one L2.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t id, uint32_t total) {
+  constexpr uint32_t kXcd = 8;
+  if (total % kXcd) return id;
+  return (id % kXcd) * (total / kXcd) + id / kXcd;
+}
+
+// Convert four consecutive fp32 values to T and store them to LDS.
+template <typename T>
+__device__ __forceinline__ void store4(T* dst, float a, float b, float c, float d) {
+  if constexpr (sizeof(T) == 2) {
+    *reinterpret_cast<u32x2*>(dst) = u32x2{pack_bf16x2(a, b), pack_bf16x2(c, d)};
+  } else {
+    *reinterpret_cast<f32x4*>(dst) = f32x4{a, b, c, d};
+  }
+}
+
+// Cooperative HBM -> register -> LDS streaming of NT row-major tiles of ROWS
+// rows x D elements by a 256-thread work-group.  issue() starts the global
+// loads (rows at or past `nrows` read as zero), commit() writes them to LDS.
+template <typename T, int D, int ROWS, int NT>
+struct TileStream {
+  using C = Cfg<T, D>;
+  static constexpr int TILE_VECS = ROWS * C::VPR;
+  static constexpr int ITERS = (TILE_VECS + 255) / 256;
+  u32x4 pre[NT][ITERS];
+
+  __device__ __forceinline__ void issue(const T* const (&src)[NT], const int64_t (&row_stride)[NT], int row0, int nrows, int tid) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int v = tid + it * 256;
+        const int row = v / C::VPR, cv = v % C::VPR;
+        const bool ok = (v < TILE_VECS) && (row0 + row < nrows);
+        pre[t][it] = ok ? *reinterpret_cast<const u32x4*>(src[t] + (int64_t)(row0 + row) * row_stride[t] + cv * C::VEC)
+                        : u32x4{0, 0, 0, 0};
+      }
+    }
+  }
+  __device__ __forceinline__ void commit(T* const (&dst)[NT], int tid) const {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int v = tid + it * 256;
+        const int row = v / C::VPR, cv = v % C::VPR;
+        if (v < TILE_VECS) *reinterpret_cast<u32x4*>(dst[t] + row * C::STRIDE + cv * C::VEC) = pre[t][it];
+      }
+    }
+  }
+};
+
+// Zero the contraction padding (vectors VPR .. 2*NCHUNK-1 of every row) of an
+// LDS tile; tile commits never touch those columns afterwards.
+template <typename T, int D, int ROWS>
+__device__ __forceinline__ void zero_tile_padding(T* tile, int tid) {
+  using C = Cfg<T, D>;
+  if constexpr (2 * C::NCHUNK > C::VPR) {
+    constexpr int PADV = 2 * C::NCHUNK - C::VPR;
+    for (int i = tid; i < ROWS * PADV; i += 256) {
+      const int row = i / PADV, cv = C::VPR + i % PADV;
+      *reinterpret_cast<u32x4*>(tile + row * C::STRIDE + cv * C::VEC) = u32x4{0, 0, 0, 0};
+    }
+  }
+}
+
+// Epilogue helper: a work-group's NDT transposed accumulator tiles (lane = output
+// row wave*32+c32, in-lane = head-dim index) are scaled, transposed through the
+// LDS staging area and stored with coalesced 16-byte rows.  Must be called by
+// all 256 threads; `stage` may alias the tile buffers (the leading barrier
+// protects them).
+template <typename T, int D, typename F>
+__device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t row_stride, int row0, int nrows, int tid, F value) {
+  using C = Cfg<T, D>;
+  const int lane = tid & 63, wave = tid >> 6, c32 = lane & 31, g = lane >> 5;
+  __syncthreads();
+  T* srow = stage + (wave * 32 + c32) * C::OSTRIDE;
+#pragma unroll
+  for (int t = 0; t < C::NDT; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      store4<T>(srow + t * 32 + j * 8 + 4 * g, value(t, 4 * j), value(t, 4 * j + 1), value(t, 4 * j + 2), value(t, 4 * j + 3));
+  __syncthreads();
+  for (int v = tid; v < 128 * C::VPR; v += 256) {
+    const int row = v / C::VPR, cv = v % C::VPR;
+    if (row0 + row < nrows)
+      *reinterpret_cast<u32x4*>(gdst + (int64_t)(row0 + row) * row_stride + cv * C::VEC) =
+          *reinterpret_cast<const u32x4*>(stage + row * C::OSTRIDE + cv * C::VEC);
+  }
+}
+
+}  // namespace dmf

@@ -1,0 +1,35 @@
+// Kernel parameter blocks and launcher prototypes shared between the C-ABI
+// translation unit and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dmf {
+
+// Strides are in elements: st[t] = {stride_B, stride_L, stride_H}; the head-dim
+// stride is 1 by contract.
+struct FwdParams {
+  const void *q, *k, *v, *tq, *tk, *tv;
+  void *o, *to;
+  float* lse;               // (B, H, Lq) or nullptr
+  float* dlse;              // (B, H, Lq) or nullptr: tangent of lse (JVP kernels only)
+  int64_t st[8][3];         // q, k, v, tq, tk, tv, o, to
+  int H, Lq, Lkv;
+  float scale, scale_log2;  // softmax scale and scale * log2(e)
+};
+
+struct BwdParams {
+  const void *dout, *q, *k, *v, *o;
+  const float* lse;         // (B, H, Lq)
+  void *dq, *dk, *dv;
+  float* delta;             // (B, H, Lq): written by the dQ kernel, read by the dK/dV kernel
+  int64_t st[8][3];         // dout, q, k, v, o, dq, dk, dv
+  int H, Lq, Lkv;
+  float scale, scale_log2;
+};
+
+// Return 0 or a negative DMF_ATTN_E* code.
+int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream);
+int launch_bwd(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream);
+
+}  // namespace dmf

@@ -1,0 +1,118 @@
+"""Forward-mode attention operator on hand-written gfx950 kernels.
+
+Host-side mirror of the reference's operator module
+(models/flash_attention_2_jvp.py:177-319): the same ``FlashAttnFunc`` protocol
+(new-style ``forward`` without ctx + ``setup_context``, as ``torch.func.jvp``
+requires) and the same ``flash_attn_func`` dual-tensor wrapper, but every
+device computation goes through the C ABI in ``dmf_amd._lib``:
+
+* dual inputs  -> one fused forward+JVP kernel (replaces the Triton
+  ``_attn_fwd_dual[_split]`` launch, reference :196-230),
+* plain inputs -> primal-only forward kernel (replaces ``flash_attn_2_cuda.fwd``,
+  reference :233-243),
+* ``backward`` -> dQ/dK/dV kernels (replaces ``flash_attn_2_cuda.bwd``,
+  reference :260-276).
+
+Unlike the reference, ``jvp`` is functional: when ``FlashAttnFunc.apply`` is
+handed dual tensors directly, the tangents of ``o`` and ``lse`` are computed by
+a second pass of the fused kernel over the saved primals.
+"""
+from __future__ import annotations
+
+import torch
+import torch.autograd.forward_ad as fwAD
+from torch._C import _functorch
+
+from . import _lib
+
+
+def _raw(t):
+    """Strip functorch wrappers: inside ``jvp`` the saved tensors and tangents
+    arrive wrapped at the transform level and have no storage of their own."""
+    while t is not None and _functorch.is_functorch_wrapped_tensor(t):
+        t = _functorch.get_unwrapped(t)
+    return t
+
+
+def _default_scale(q: torch.Tensor, softmax_scale):
+    return q.shape[-1] ** (-0.5) if softmax_scale is None else softmax_scale
+
+
+class FlashAttnFunc(torch.autograd.Function):
+    """(q, k, v, tq, tk, tv, softmax_scale) -> (o, lse, to); tensors are (B, L, H, D).
+
+    ``lse`` is the natural-log logsumexp of the scaled scores, (B, H, Lq) fp32.
+    ``to`` is None when any tangent is None.
+    """
+
+    @staticmethod
+    def forward(q, k, v, tq, tk, tv, softmax_scale):
+        scale = _default_scale(q, softmax_scale)
+        enable_jvp = (tq is not None) and (tk is not None) and (tv is not None)
+        if enable_jvp:
+            o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)
+        else:
+            o, lse = _lib.fwd(q, k, v, scale, need_lse=True)
+            to = None
+        return o, lse, to
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        q, k, v, tq, tk, tv, softmax_scale = inputs
+        o, lse, to = outputs
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.save_for_forward(q, k, v)
+        ctx.softmax_scale = _default_scale(q, softmax_scale)
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, dout, *ignored):
+        # Gradients flow through the primal output only: cotangents of ``lse``
+        # and ``to`` are dropped and the tangent inputs get no gradient, exactly
+        # as in the reference (flash_attention_2_jvp.py:260-276) -- valid for the
+        # MeanFlow loss because its JVP target is detached (loss.py:171-172).
+        q, k, v, o, lse = ctx.saved_tensors
+        if dout is None:
+            return None, None, None, None, None, None, None
+        dq, dk, dv = _lib.bwd(dout, q, k, v, o, lse, ctx.softmax_scale)
+        return dq, dk, dv, None, None, None, None
+
+    @staticmethod
+    def jvp(ctx, gq, gk, gv, *ignored):
+        # Tangents of ``o`` and ``lse`` along (gq, gk, gv) from a second pass of
+        # the fused kernel.  ``to`` (if any) gets no tangent: that would be a
+        # second-order quantity, which the reference does not provide either.
+        if gq is None and gk is None and gv is None:
+            return None, None, None
+        q, k, v = (_raw(t) for t in ctx.saved_tensors[:3])
+        gq, gk, gv = _raw(gq), _raw(gk), _raw(gv)
+        gq = torch.zeros_like(q) if gq is None else gq
+        gk = torch.zeros_like(k) if gk is None else gk
+        gv = torch.zeros_like(v) if gv is None else gv
+        _, to, _, dlse = _lib.fwd_jvp(q, k, v, gq, gk, gv, ctx.softmax_scale, need_dlse=True)
+        return to, dlse, None
+
+
+def _is_dual_mode(*tensors) -> bool:
+    """True if any tensor carries a forward-AD tangent (reference :285-291)."""
+    return any(fwAD.unpack_dual(t).tangent is not None for t in tensors)
+
+
+def flash_attn_func(q, k, v, softmax_scale=None):
+    """Attention on (B, L, H, D) tensors; dual tensors in -> dual tensor out.
+
+    Same contract as the reference's ``flash_attn_func``
+    (models/flash_attention_2_jvp.py:294-319): under forward-mode AD the
+    primals and tangents are unpacked (a missing tangent becomes zeros, :303-304),
+    pushed through one fused kernel, and re-packed with ``fwAD.make_dual``.
+    """
+    if _is_dual_mode(q, k, v):
+        primals, tangents = [], []
+        for t in (q, k, v):
+            p, tg = fwAD.unpack_dual(t)
+            primals.append(p)
+            tangents.append(torch.zeros_like(p) if tg is None else tg)
+        out, _, t_out = FlashAttnFunc.apply(*primals, *tangents, softmax_scale)
+        return fwAD.make_dual(out, t_out)
+    out, _, _ = FlashAttnFunc.apply(q, k, v, None, None, None, softmax_scale)
+    return out

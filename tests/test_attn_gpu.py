@@ -1,0 +1,230 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI (dmf_amd._lib is
+a 1:1 ctypes binding of include/dmf_attn.h), against the CPU oracle -- the
+reference's naive 'base' attention under torch.func.jvp in fp32 on the same
+seeded inputs.
+
+Tolerances (relative L2 over the whole tensor), from the contract of this build:
+    fp32 mode: 1e-5      bf16 mode: 2e-2
+for O, dO and for dQ, dK, dV.  In bf16 mode the oracle sees the bf16-rounded
+inputs (the values the kernel sees), computed in fp32.
+"""
+import pytest
+import torch
+
+from dmf_amd import _lib, flash_attn_func, FlashAttnFunc, attn_op
+from dmf_amd.layers import Attention
+from oracle import attn_oracle as ao
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+DEV = "cuda:0"
+
+
+def _case(B, L, H, D, dtype, seed, std=1.0, Lkv=None):
+    """Seeded CPU inputs rounded to `dtype`, their fp32 view for the oracle and
+    their device copies."""
+    cpu = [t.to(dtype) for t in ao.make_inputs(B, L, H, D, seed, std=std, Lkv=Lkv)]
+    ref = [t.float() for t in cpu]
+    dev = [t.to(DEV) for t in cpu]
+    return ref, dev
+
+
+def _check(name, got, exp, tol):
+    err = ao.rel_l2(got.float().cpu(), exp)
+    assert err <= tol, f"{name}: rel-L2 {err:.3e} > {tol:.1e}"
+    return err
+
+
+def _parity(B, L, H, D, dtype, seed, std=1.0, Lkv=None, bwd=True):
+    print(f"case B{B} L{L} Lkv{Lkv} H{H} D{D} {dtype} seed{seed}", flush=True)
+    tol = TOL[dtype]
+    (q, k, v, tq, tk, tv, do), (gq, gk, gv, gtq, gtk, gtv, gdo) = _case(B, L, H, D, dtype, seed, std, Lkv)
+    scale = D ** -0.5
+    o_ref, to_ref = ao.base_attn_jvp(q, k, v, tq, tk, tv)
+    lse_ref = ao.lse_ref(q, k)
+    # fused forward + JVP
+    o, to, lse, dlse = _lib.fwd_jvp(gq, gk, gv, gtq, gtk, gtv, scale, need_dlse=True)
+    _check("o (fwd+jvp)", o, o_ref, tol)
+    _check("to", to, to_ref, tol)
+    _check("lse", lse, lse_ref, 1e-5 if dtype == torch.float32 else 1e-3)
+    cf_mu = torch.from_numpy(ao.closed_form_fp64(q, k, v, tq, tk, tv)["mu"])
+    _check("dlse", dlse, cf_mu, tol)
+    # primal-only forward
+    o2, lse2 = _lib.fwd(gq, gk, gv, scale)
+    _check("o (fwd)", o2, o_ref, tol)
+    _check("lse (fwd)", lse2, lse_ref, 1e-5 if dtype == torch.float32 else 1e-3)
+    o3, none = _lib.fwd(gq, gk, gv, scale, need_lse=False)
+    assert none is None and torch.equal(o3, o2)
+    if bwd:
+        dq_ref, dk_ref, dv_ref = ao.base_attn_grads(q, k, v, do)
+        dq, dk, dv = _lib.bwd(gdo, gq, gk, gv, o2, lse2, scale)
+        _check("dq", dq, dq_ref, tol)
+        _check("dk", dk, dk_ref, tol)
+        _check("dv", dv, dv_ref, tol)
+
+
+# ---- BASELINE configurations at sizes the oracle finishes in seconds -------
+def test_config1_fp32():
+    """Config 1: B=2, H=12, N=256, D=64, fp32, N(0,1), seed 1."""
+    _parity(2, 256, 12, 64, torch.float32, seed=1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L", [256, 1024])
+def test_xl2_shape_reduced_batch(L, dtype):
+    """Configs 3/4 shape (H=16, D=72) with a batch the CPU oracle can follow."""
+    _parity(2 if L == 256 else 1, L, 16, 72, dtype, seed=3 if L == 256 else 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 64, 72, 80, 96, 128])
+def test_all_head_dims(D, dtype):
+    _parity(1, 192, 3, D, dtype, seed=10 + D)
+
+
+# ---- the reference self-test family: b=2, N(0, 0.5^2), bf16 -----------------
+# (models/flash_attention_2_jvp.py:339-353; a diagonal of its l x h x d grid so
+# the CPU oracle stays within seconds; its tolerance atol=1.2e-3 is checked too)
+@pytest.mark.parametrize("l,h,d", [(256, 16, 64), (256, 24, 72), (256, 32, 96), (256, 16, 128),
+                                   (1024, 16, 72), (1024, 24, 64), (2048, 16, 72), (1024, 16, 128)])
+def test_reference_family(l, h, d):
+    dtype = torch.bfloat16
+    print(f"case ref-family l{l} h{h} d{d}", flush=True)
+    (q, k, v, tq, tk, tv, do), dev = _case(2, l, h, d, dtype, seed=l + h + d, std=0.5)
+    gq, gk, gv, gtq, gtk, gtv, gdo = dev
+    gq, gk, gv = (t.requires_grad_() for t in (gq, gk, gv))
+    u, du = torch.func.jvp(flash_attn_func, (gq, gk, gv), (gtq, gtk, gtv))
+    dq, dk, dv = torch.autograd.grad(u, (gq, gk, gv), gdo)
+    u_ref, du_ref = ao.base_attn_jvp(q, k, v, tq, tk, tv, fn=ao.raw_attn)
+    dq_ref, dk_ref, dv_ref = ao.base_attn_grads(q, k, v, do, fn=ao.raw_attn)
+    for name, got, exp in (("u", u, u_ref), ("du", du, du_ref), ("dq", dq, dq_ref), ("dk", dk, dk_ref), ("dv", dv, dv_ref)):
+        _check(name, got, exp, 2e-2)
+        # reference tolerance: atol 1.2e-3 against a bf16 result; ours is compared
+        # with the fp32 oracle, so allow the bf16 rounding of the value itself too
+        diff = (got.float().cpu() - exp).abs()
+        assert bool((diff <= 1.2e-3 + exp.abs() * 2 ** -8).all()), f"{name}: max abs diff {diff.max():.3e}"
+
+
+# ---- edge cases: ragged and tiny sequences, cross-attention lengths --------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("Lq,Lkv", [(1, 1), (16, 16), (64, 64), (100, 77), (129, 65), (257, 300), (128, 33)])
+def test_ragged_lengths(Lq, Lkv, dtype):
+    _parity(2, Lq, 2, 72, dtype, seed=Lq * 7 + Lkv, Lkv=Lkv)
+
+
+def test_packed_qkv_strided_views_match_contiguous():
+    """q, k, v (and tangents) as views into a packed (B, L, 3, H, D) buffer with
+    strides (3LHD, 3HD, D, 1), the layout models/layers.py:143-147 produces."""
+    B, L, H, D = 2, 256, 4, 72
+    for dtype in (torch.float32, torch.bfloat16):
+        g = torch.Generator().manual_seed(5)
+        qkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(DEV)
+        tqkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(DEV)
+        q, k, v = qkv.permute(2, 0, 1, 3, 4).unbind(0)
+        tq, tk, tv = tqkv.permute(2, 0, 1, 3, 4).unbind(0)
+        assert q.stride() == (3 * L * H * D, 3 * H * D, D, 1)
+        a = _lib.fwd_jvp(q, k, v, tq, tk, tv, D ** -0.5)
+        b = _lib.fwd_jvp(*(t.contiguous() for t in (q, k, v, tq, tk, tv)), D ** -0.5)
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+        do = torch.randn(B, L, H, D, generator=g).to(dtype).to(DEV)
+        ga = _lib.bwd(do, q, k, v, a[0], a[2], D ** -0.5)
+        gb = _lib.bwd(do, q.contiguous(), k.contiguous(), v.contiguous(), a[0], a[2], D ** -0.5)
+        for x, y in zip(ga, gb):
+            assert torch.equal(x, y)
+
+
+# ---- full BASELINE sizes through size-independent properties ---------------
+@pytest.mark.parametrize("B,L", [(256, 256), (64, 1024)])
+def test_full_size_properties(B, L):
+    """Configs 3 (B256 N256) and 4 (B64 N1024, qk-norm) at full size, bf16:
+    slices of (b, h) units against the oracle, plus properties that hold at any
+    size: dQ=dK=0 => dO = Attn(Q, K, dV); linearity in the tangents; the
+    adjoint identity <JVP t, w> = <t, VJP w>."""
+    H, D, dtype = 16, 72, torch.bfloat16
+    g = torch.Generator(device=DEV).manual_seed(B + L)
+    q, k, v, tq, tk, tv, do = (torch.randn(B, L, H, D, generator=g, device=DEV, dtype=torch.float32) for _ in range(7))
+    if L == 1024:   # config 4: q, k RMS-normalised per head, gain 1
+        q, k = ao.rms_norm(q), ao.rms_norm(k)
+    q, k, v, tq, tk, tv, do = (t.to(dtype) for t in (q, k, v, tq, tk, tv, do))
+    scale = D ** -0.5
+    o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)
+    # (1) sampled units against the oracle
+    for b, h in ((0, 0), (B // 2, 7), (B - 1, H - 1)):
+        sl = lambda t: t[b:b + 1, :, h:h + 1].float().cpu()
+        o_ref, to_ref = ao.base_attn_jvp(*(sl(t) for t in (q, k, v, tq, tk, tv)))
+        _check(f"o[{b},{h}]", sl(o), o_ref, 2e-2)
+        _check(f"to[{b},{h}]", sl(to), to_ref, 2e-2)
+    # (2) dQ = dK = 0  =>  dO = Attn(Q, K, dV), bit-for-bit the same products
+    z = torch.zeros_like(q)
+    _, to_v, _ = _lib.fwd_jvp(q, k, v, z, z, tv, scale)
+    o_tv, _ = _lib.fwd(q, k, tv, scale)
+    _check("dQ=dK=0", to_v, o_tv.float().cpu(), 1e-2)
+    # (3) linearity: JVP(2a - 3b) = 2 JVP(a) - 3 JVP(b)
+    _, to_b, _ = _lib.fwd_jvp(q, k, v, tk, tq, do, scale)       # another tangent triple
+    _, to_c, _ = _lib.fwd_jvp(q, k, v, (2 * tq.float() - 3 * tk.float()).to(dtype), (2 * tk.float() - 3 * tq.float()).to(dtype),
+                              (2 * tv.float() - 3 * do.float()).to(dtype), scale)
+    _check("linearity", to_c, (2 * to.float() - 3 * to_b.float()).cpu(), 3e-2)
+    # (4) adjoint identity ties the backward to the tangent
+    dq, dk, dv = _lib.bwd(do, q, k, v, o, lse, scale)
+    lhs = (to.double() * do.double()).sum().item()
+    rhs = sum((a.double() * b.double()).sum().item() for a, b in ((tq, dq), (tk, dk), (tv, dv)))
+    norm = (to.double().norm() * do.double().norm()).item()
+    assert abs(lhs - rhs) / norm < 2e-3, (lhs, rhs, norm)
+    # (5) outputs are finite and the primal-only kernel agrees with the fused one
+    o2, lse2 = _lib.fwd(q, k, v, scale)
+    assert torch.isfinite(o).all() and torch.isfinite(to).all() and torch.isfinite(dq).all()
+    _check("o fused vs primal-only", o, o2.float().cpu(), 1e-3)
+    _check("lse fused vs primal-only", lse, lse2.float().cpu(), 1e-6)
+
+
+# ---- the operator as the model calls it -------------------------------------
+def test_attn_op_hip_under_func_jvp_and_backward():
+    B, L, H, D = 2, 256, 4, 64
+    (q, k, v, tq, tk, tv, do), dev = _case(B, L, H, D, torch.float32, seed=21)
+    gq, gk, gv, gtq, gtk, gtv, gdo = dev
+    gq, gk, gv = (t.requires_grad_() for t in (gq, gk, gv))
+    f = lambda a, b, c: attn_op(a, b, c, op="hip")
+    u, du = torch.func.jvp(f, (gq, gk, gv), (gtq, gtk, gtv))
+    u_ref, du_ref = ao.base_attn_jvp(q, k, v, tq, tk, tv)
+    _check("u", u, u_ref, 1e-5)
+    _check("du", du, du_ref, 1e-5)
+    grads = torch.autograd.grad(u, (gq, gk, gv), gdo)
+    for name, got, exp in zip(("dq", "dk", "dv"), grads, ao.base_attn_grads(q, k, v, do)):
+        _check(name, got, exp, 1e-5)
+    # no-grad / plain path and the Function's own jvp (second pass)
+    with torch.no_grad():
+        _check("plain", attn_op(gq, gk, gv, op="hip"), u_ref, 1e-5)
+    h = lambda a, b, c: FlashAttnFunc.apply(a, b, c, None, None, None, None)[:2]
+    (o2, lse2), (to2, dlse2) = torch.func.jvp(h, (gq.detach(), gk.detach(), gv.detach()), (gtq, gtk, gtv))
+    _check("Function.jvp to", to2, du_ref, 1e-5)
+    _check("Function.jvp dlse", dlse2, torch.from_numpy(ao.closed_form_fp64(q, k, v, tq, tk, tv)["mu"]), 1e-5)
+
+
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_attention_module_hip_vs_base(qk_norm):
+    """The Attention layer (models/layers.py:119-154 restated) with op 'hip'
+    against the same layer with op 'base', same weights, under torch.func.jvp."""
+    torch.manual_seed(0)
+    C, H, B, L = 288, 4, 2, 256
+    m_hip = Attention(C, num_heads=H, qkv_bias=True, qk_norm=qk_norm, attn_func="hip").to(DEV)
+    m_base = Attention(C, num_heads=H, qkv_bias=True, qk_norm=qk_norm, attn_func="base").to(DEV)
+    m_base.load_state_dict(m_hip.state_dict())
+    x, tx = torch.randn(B, L, C, device=DEV), torch.randn(B, L, C, device=DEV)
+    y, ty = torch.func.jvp(m_hip, (x,), (tx,))
+    y_ref, ty_ref = torch.func.jvp(m_base, (x,), (tx,))
+    _check("y", y, y_ref.cpu(), 2e-5)
+    _check("ty", ty, ty_ref.cpu(), 2e-5)
+    y.square().sum().backward()
+    y_ref.square().sum().backward()
+    for (n, p), (_, pr) in zip(m_hip.named_parameters(), m_base.named_parameters()):
+        _check(f"grad {n}", p.grad, pr.grad.cpu(), 5e-5)
+
+
+def test_unsupported_head_dim_raises():
+    q = torch.randn(1, 16, 2, 40, device=DEV)
+    with pytest.raises(RuntimeError, match="head dim"):
+        flash_attn_func(q, q, q)
+    with pytest.raises(TypeError):
+        flash_attn_func(q.half(), q.half(), q.half())

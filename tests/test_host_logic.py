@@ -1,0 +1,186 @@
+"""CPU-only tests: the C-ABI library loads and exports what include/dmf_attn.h
+declares, argument validation returns the documented codes (no kernel is
+launched on those paths), and the autograd / forward-AD protocol of the Python
+operator behaves like the reference's (models/flash_attention_2_jvp.py:177-319)
+when the three kernel calls are replaced by stand-ins defined in this file."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import dmf_amd
+from dmf_amd import _lib, flash_attention_hip_jvp as fa
+from dmf_amd.layers import attn_op, Attention, RMSNorm, get_2d_sincos_pos_embed
+from oracle import attn_oracle as ao
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "dmf_attn.h")).read()
+    return re.findall(r"DMF_ATTN_API\s+[\w\s\*]+?\b(dmf_attn_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert set(names) == set(_lib.SIGNATURES), names
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.dmf_attn_version() >= 1
+    assert lib.dmf_attn_strerror(0) == b"ok"
+    for code in range(-7, 0):
+        assert b"unknown" not in lib.dmf_attn_strerror(code)
+    assert b"unknown" in lib.dmf_attn_strerror(-99)
+
+
+def test_validation_codes_without_launch():
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096 + 16)
+    p = (ctypes.addressof(buf) + 15) // 16 * 16
+    st4 = (ctypes.c_int64 * 16)(*([64 * 4 * 2, 64 * 2, 64, 1] * 4))
+    call = lambda **kw: lib.dmf_attn_fwd(
+        kw.get("q", p), p, p, p, None, kw.get("st", st4), kw.get("B", 1), 2, 4, 4, kw.get("D", 64), 0.125, kw.get("dtype", 0), None)
+    assert call(D=40) == -2          # head dim
+    assert call(dtype=7) == -1       # dtype
+    assert call(B=0) == -3           # shape
+    assert call(q=None) == -5        # null
+    assert call(q=p + 4) == -6       # alignment
+    bad = (ctypes.c_int64 * 16)(*([64 * 4 * 2, 64 * 2, 64, 2] * 4))
+    assert call(st=bad) == -4        # last-dim stride
+    bad2 = (ctypes.c_int64 * 16)(*([64 * 4 * 2, 64 * 2 + 1, 64, 1] * 4))
+    assert call(st=bad2) == -4       # row alignment
+    # fwd_jvp requires lse
+    st8 = (ctypes.c_int64 * 32)(*([64 * 4 * 2, 64 * 2, 64, 1] * 8))
+    assert lib.dmf_attn_fwd_jvp(p, p, p, p, p, p, p, p, None, None, st8, 1, 2, 4, 4, 64, 0.125, 0, None) == -5
+    assert lib.dmf_attn_bwd(p, p, p, p, p, None, p, p, p, None, st8, 1, 2, 4, 4, 64, 0.125, 0, None) == -5
+
+
+def test_cpu_tensors_fail_loudly():
+    q = torch.randn(1, 4, 2, 64)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        dmf_amd.flash_attn_func(q, q, q)
+    with pytest.raises(ValueError):
+        attn_op(q, q, q, op="nope")
+
+
+@pytest.fixture
+def fake_kernels(monkeypatch):
+    """Replace the three C-ABI calls by plain-torch stand-ins and count calls."""
+    calls = {"fwd": 0, "fwd_jvp": 0, "bwd": 0}
+
+    def fwd(q, k, v, scale, need_lse=True):
+        calls["fwd"] += 1
+        return ao.base_attn(q, k, v).contiguous(), ao.lse_ref(q, k, scale).float()
+
+    def fwd_jvp(q, k, v, tq, tk, tv, scale, need_dlse=False):
+        calls["fwd_jvp"] += 1
+        # plain torch ops only: this runs inside forward-AD / functorch levels
+        o, to, lse, mu = ao.streaming_fwd_jvp(q, k, v, tq, tk, tv, scale=scale, block_kv=8, dtype=q.dtype)
+        out = (o.contiguous(), to.contiguous(), lse.float())
+        return out + (mu.float(),) if need_dlse else out
+
+    def bwd(dout, q, k, v, o, lse, scale):
+        calls["bwd"] += 1
+        with torch.enable_grad():   # autograd runs backward() with grad mode off
+            return ao.base_attn_grads(q, k, v, dout)
+
+    monkeypatch.setattr(_lib, "fwd", fwd)
+    monkeypatch.setattr(_lib, "fwd_jvp", fwd_jvp)
+    monkeypatch.setattr(_lib, "bwd", bwd)
+    return calls
+
+
+def test_func_jvp_then_backward_protocol(fake_kernels):
+    """Structure of the reference self-test (flash_attention_2_jvp.py:344-376):
+    jvp of the op, then backward on the primal output."""
+    q, k, v, tq, tk, tv, do = [t.double() for t in ao.make_inputs(2, 16, 2, 8, seed=3, std=0.5)]
+    q, k, v = (t.requires_grad_() for t in (q, k, v))
+    u_ref, du_ref = torch.func.jvp(ao.raw_attn, (q, k, v), (tq, tk, tv))
+    u, du = torch.func.jvp(fa.flash_attn_func, (q, k, v), (tq, tk, tv))
+    assert fake_kernels == {"fwd": 0, "fwd_jvp": 1, "bwd": 0}     # one fused pass, no separate primal pass
+    assert ao.rel_l2(u, u_ref) < 1e-12 and ao.rel_l2(du, du_ref) < 1e-12
+    ref = torch.autograd.grad(u_ref, (q, k, v), do)
+    got = torch.autograd.grad(u, (q, k, v), do)
+    assert fake_kernels["bwd"] == 1
+    for a, b in zip(got, ref):
+        assert ao.rel_l2(a, b) < 1e-12
+
+
+def test_partial_tangents_are_zero_filled(fake_kernels):
+    """Only q is dual: k, v tangents become zeros (flash_attention_2_jvp.py:303-304)."""
+    import torch.autograd.forward_ad as fwAD
+    q, k, v, tq, *_ = [t.double() for t in ao.make_inputs(1, 12, 2, 8, seed=4)]
+    with fwAD.dual_level():
+        out = fa.flash_attn_func(fwAD.make_dual(q, tq), k, v)
+        o, to = fwAD.unpack_dual(out)
+    _, to_ref = ao.base_attn_jvp(q, k, v, tq, torch.zeros_like(k), torch.zeros_like(v))
+    assert ao.rel_l2(to, to_ref) < 1e-12
+    assert fake_kernels["fwd_jvp"] == 1
+
+
+def test_plain_inputs_take_primal_only_path(fake_kernels):
+    q, k, v, *_ = [t.double() for t in ao.make_inputs(1, 12, 2, 8, seed=5)]
+    with torch.no_grad():
+        o = fa.flash_attn_func(q, k, v)
+    assert fake_kernels == {"fwd": 1, "fwd_jvp": 0, "bwd": 0}
+    assert ao.rel_l2(o, ao.base_attn(q, k, v)) < 1e-12
+    q.requires_grad_()
+    o = fa.flash_attn_func(q, k, v)
+    o.sum().backward()
+    assert fake_kernels["bwd"] == 1 and q.grad is not None
+
+
+def test_function_jvp_staticmethod_is_functional(fake_kernels):
+    """Dual tensors handed straight to FlashAttnFunc.apply: forward runs
+    primal-only, then ``jvp`` produces the tangent with a second fused pass."""
+    q, k, v, tq, tk, tv, _ = [t.double() for t in ao.make_inputs(1, 12, 2, 8, seed=6)]
+    f = lambda q, k, v: fa.FlashAttnFunc.apply(q, k, v, None, None, None, None)[0]
+    o, to = torch.func.jvp(f, (q, k, v), (tq, tk, tv))
+    o_ref, to_ref = ao.base_attn_jvp(q, k, v, tq, tk, tv)
+    assert ao.rel_l2(o, o_ref) < 1e-12 and ao.rel_l2(to, to_ref) < 1e-12
+    assert fake_kernels["fwd"] == 1 and fake_kernels["fwd_jvp"] == 1
+    # the lse output carries its tangent too (rowsum(P*dS))
+    g = lambda q, k, v: fa.FlashAttnFunc.apply(q, k, v, None, None, None, None)[1]
+    lse, dlse = torch.func.jvp(g, (q, k, v), (tq, tk, tv))
+    cf = ao.closed_form_fp64(q, k, v, tq, tk, tv)
+    assert ao.rel_l2(lse, torch.from_numpy(cf["lse"])) < 1e-6 and ao.rel_l2(dlse, torch.from_numpy(cf["mu"])) < 1e-6
+
+
+def test_attn_op_base_and_sdpa_branches():
+    q, k, v, *_ = ao.make_inputs(2, 10, 3, 16, seed=7)
+    assert ao.rel_l2(attn_op(q, k, v, "base"), ao.base_attn(q, k, v)) < 1e-7
+    assert ao.rel_l2(attn_op(q, k, v, "torch_sdpa"), ao.base_attn(q, k, v)) < 2e-6
+
+
+def test_attention_module_feeds_packed_qkv_views(fake_kernels, monkeypatch):
+    """q, k, v reach the operator as (B, L, H, D) views with strides
+    (3LHD, 3HD, D, 1) (reference models/layers.py:143-147); with qk-norm q and k
+    become contiguous and v stays a view."""
+    seen = []
+    orig = _lib.fwd
+    monkeypatch.setattr(_lib, "fwd", lambda q, k, v, s, need_lse=True: (seen.append((q.stride(), k.stride(), v.stride())), orig(q, k, v, s))[1])
+    B, L, H, D = 2, 6, 3, 8
+    x = torch.randn(B, L, H * D)
+    for qk_norm in (False, True):
+        m = Attention(H * D, num_heads=H, qkv_bias=True, qk_norm=qk_norm, attn_func="hip")
+        m_ref = Attention(H * D, num_heads=H, qkv_bias=True, qk_norm=qk_norm, attn_func="base")
+        m_ref.load_state_dict(m.state_dict())
+        with torch.no_grad():
+            assert ao.rel_l2(m(x), m_ref(x)) < 1e-5
+    packed = (3 * L * H * D, 3 * H * D, D, 1)
+    assert seen[0] == (packed, packed, packed)
+    assert seen[1][2] == packed and seen[1][0] == (L * H * D, H * D, D, 1)
+
+
+def test_rmsnorm_and_pos_embed_match_oracle_formulas():
+    x = torch.randn(2, 5, 3, 72)
+    assert ao.rel_l2(RMSNorm(72)(x), ao.rms_norm(x)) < 1e-7
+    pe = get_2d_sincos_pos_embed(16, 4)
+    assert pe.shape == (16, 16)
+    # token (row r, col c) -> first half encodes c, second half r; position 0 -> sin 0, cos 1
+    assert abs(pe[0, :4]).max() == 0 and (pe[0, 4:8] == 1).all()
+    assert pe[1, 0] == pytest.approx(float(torch.sin(torch.tensor(1.0))))   # token 1 = (row 0, col 1)
+    assert pe[4, 8] == pytest.approx(float(torch.sin(torch.tensor(1.0))))   # token 4 = (row 1, col 0)
