@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the forward-mode attention hot path on one MI355X.
+
+A "step" is one launch of the fused forward+JVP kernel over one synthetic batch
+of the headline workload (SiT/DMFT-XL/2 at 512px: B=64, H=16, N=1024, D=72,
+bf16, q/k RMS-normalised), inputs resident in HBM.  Prints ONE JSON line:
+
+  metric/value   attention fwd+JVP TFLOP/s on the algorithmic FLOP count
+                 12*B*H*N^2*D (unpadded head dim)
+  roofline       the same figure against MI355X's dense bf16 MFMA peak
+  cpu_baseline   the CPU oracle ('base' attention under torch.func.jvp, fp32)
+                 timed on this box's host cores on a bounded slice of the
+                 same workload
+  extra          the other kernel-level figures (N=256 shape, backward,
+                 primal-only forward) and DMFT forward+JVP images/s
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, H, N, D, qk_norm)
+    "xl2_512px": (64, 16, 1024, 72, True),    # BASELINE config 4 (headline)
+    "xl2_256px": (256, 16, 256, 72, False),   # BASELINE config 3
+}
+
+
+def make_inputs(name, device, dtype, seed):
+    import torch
+    from dmf_amd.layers import RMSNorm
+
+    B, H, N, D, qk_norm = WORKLOADS[name]
+    g = torch.Generator(device=device).manual_seed(seed)
+    q, k, v, tq, tk, tv, do = (torch.randn(B, N, H, D, generator=g, device=device, dtype=torch.float32) for _ in range(7))
+    if qk_norm:
+        norm = RMSNorm(D).to(device)
+        with torch.no_grad():
+            q, k = norm(q), norm(k)
+    return [t.to(dtype).contiguous() for t in (q, k, v, tq, tk, tv, do)]
+
+
+def time_gpu(fn, steps, warmup):
+    """Average duration (ms) of `fn` over `steps` back-to-back launches on the
+    current stream, HIP events bracketing the timed region."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return start.elapsed_time(stop) / steps, wall_ms / steps
+
+
+def attn_flops(B, H, N, D, kind):
+    mult = {"fwd_jvp": 12, "fwd": 4, "bwd": 10}[kind]
+    return mult * B * H * N * N * D
+
+
+def attn_bytes(B, H, N, D, kind, elem=2):
+    if kind == "fwd_jvp":
+        return 8 * B * N * H * D * elem + 4 * B * H * N
+    if kind == "fwd":
+        return 4 * B * N * H * D * elem + 4 * B * H * N
+    return 8 * B * N * H * D * elem + 2 * 4 * B * H * N
+
+
+def cpu_baseline(name, budget_s=15.0):
+    """Oracle ('base' attention under torch.func.jvp, fp32) on the host cores,
+    on a slice of `name`: one batch element, all heads."""
+    import torch
+    from oracle import attn_oracle as ao
+
+    B, H, N, D, qk_norm = WORKLOADS[name]
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    q, k, v, tq, tk, tv, _ = ao.make_inputs(1, N, H, D, seed=4)
+    if qk_norm:
+        q, k = ao.rms_norm(q), ao.rms_norm(k)
+    ao.base_attn_jvp(q, k, v, tq, tk, tv)  # warm-up
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        ao.base_attn_jvp(q, k, v, tq, tk, tv)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    flops = attn_flops(1, H, N, D, "fwd_jvp")
+    return {
+        "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{name} slice B=1 H={H} N={N} D={D} fp32, naive attention under torch.func.jvp, "
+                  f"median of {len(times)} calls ({med * 1e3:.1f} ms/call)",
+    }
+
+
+def cpu_baseline_config1():
+    """BASELINE config 1 (B2 H12 N256 D64 fp32) at all cores and at the 4
+    intra-op threads the reference pins (train_dmf.py:33-34)."""
+    import torch
+    from oracle import attn_oracle as ao
+
+    out = {}
+    q, k, v, tq, tk, tv, _ = ao.make_inputs(2, 256, 12, 64, seed=1)
+    flops = attn_flops(2, 12, 256, 64, "fwd_jvp")
+    for label, nthr in (("all_cores", os.cpu_count() or 1), ("threads_4", 4)):
+        torch.set_num_threads(nthr)
+        for _ in range(3):
+            ao.base_attn_jvp(q, k, v, tq, tk, tv)
+        ts = []
+        for _ in range(15):
+            t0 = time.perf_counter()
+            ao.base_attn_jvp(q, k, v, tq, tk, tv)
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        out[label] = {"threads": nthr, "ms_median": ts[len(ts) // 2] * 1e3, "ms_min": ts[0] * 1e3,
+                      "gflops": flops / ts[len(ts) // 2] / 1e9}
+    torch.set_num_threads(os.cpu_count() or 1)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="xl2_512px", choices=list(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the attention units (b, h) are independent and shard "
+                 "over GPUs by batch without any collective); run with --gpus 1")
+
+    import torch
+    from dmf_amd import _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP kernels are the only implementation")
+    _lib.load()
+    dev, dtype = "cuda:0", torch.bfloat16
+    name = args.workload
+    B, H, N, D, _ = WORKLOADS[name]
+    q, k, v, tq, tk, tv, do = make_inputs(name, dev, dtype, seed=4)
+    scale = D ** -0.5
+
+    ms, wall_ms = time_gpu(lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale), args.steps, args.warmup)
+    flops = attn_flops(B, H, N, D, "fwd_jvp")
+    tflops = flops / (ms * 1e-3) / 1e12
+    result = {
+        "metric": "attn_fwd_jvp_tflops", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{name}: attention fwd+JVP B={B} H={H} N={N} D={D} bf16"
+                               + (" q,k RMS-normalised" if WORKLOADS[name][4] else ""),
+                   "flops_per_step": flops, "hbm_bytes_per_step": attn_bytes(B, H, N, D, "fwd_jvp"),
+                   "wall_ms_per_step": wall_ms},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "attn_fwd_kernel<bf16, 72, JVP>",
+                     "hbm_gbs_algorithmic": attn_bytes(B, H, N, D, "fwd_jvp") / (ms * 1e-3) / 1e9},
+    }
+
+    if not args.no_extra:
+        extra = {}
+        o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)
+        for wname in WORKLOADS:
+            Bw, Hw, Nw, Dw, _ = WORKLOADS[wname]
+            if wname == name:
+                ins, ow, lsew = (q, k, v, tq, tk, tv, do), o, lse
+            else:
+                ins = make_inputs(wname, dev, dtype, seed=3)
+                ow, _, lsew = _lib.fwd_jvp(*ins[:6], scale)
+            qw, kw, vw, tqw, tkw, tvw, dow = ins
+            row = {}
+            for kind, fn in (("fwd_jvp", lambda: _lib.fwd_jvp(qw, kw, vw, tqw, tkw, tvw, scale)),
+                             ("fwd", lambda: _lib.fwd(qw, kw, vw, scale)),
+                             ("bwd", lambda: _lib.bwd(dow, qw, kw, vw, ow, lsew, scale))):
+                t_ms, _ = time_gpu(fn, max(10, args.steps // 2), 5)
+                fl, by = attn_flops(Bw, Hw, Nw, Dw, kind), attn_bytes(Bw, Hw, Nw, Dw, kind)
+                row[kind] = {"ms": t_ms, "tflops": fl / t_ms / 1e9, "pct_bf16_mfma_peak": 100 * fl / t_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
+                             "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS}
+            extra[wname] = row
+            del ins
+        try:
+            from dmf_amd import harness
+            extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10))
+        except ImportError:
+            pass
+        result["extra"] = extra
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(name)
+        if not args.no_extra:
+            result["extra"]["cpu_config1"] = cpu_baseline_config1()
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -11,6 +11,7 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 
 import torch
+from torch._C import _functorch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdmf_attn.so")
@@ -62,12 +63,26 @@ def _dtype_code(t: torch.Tensor) -> int:
     raise TypeError(f"dmf_amd attention supports float32 and bfloat16, got {t.dtype}")
 
 
+def _raw(t):
+    """Strip functorch wrappers.  Inside a functorch transform (e.g. the ``jvp``
+    staticmethod of an autograd.Function under ``torch.func.jvp``) saved tensors
+    and even freshly allocated ones are wrapper tensors without storage."""
+    while t is not None and _functorch.is_functorch_wrapped_tensor(t):
+        t = _functorch.get_unwrapped(t)
+    return t
+
+
+def _empty(shape, dtype, device) -> torch.Tensor:
+    return _raw(torch.empty(shape, dtype=dtype, device=device))
+
+
 def _prep(t: torch.Tensor) -> torch.Tensor:
     """Kernels need unit last-dim stride and 16-byte aligned rows; views into a
     packed qkv buffer already satisfy this and are passed through untouched."""
+    t = _raw(t)
     eb = t.element_size()
     ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all((s * eb) % 16 == 0 for s in t.stride()[:-1])
-    return t if ok else t.contiguous()
+    return t if ok else _raw(t.contiguous())
 
 
 def _strides(*tensors) -> ctypes.Array:
@@ -98,10 +113,10 @@ def fwd_jvp(q, k, v, tq, tk, tv, scale: float, need_dlse: bool = False):
     q, k, v, tq, tk, tv = map(_prep, (q, k, v, tq, tk, tv))
     B, Lq, H, D = q.shape
     Lkv = k.shape[1]
-    o = torch.empty((B, Lq, H, D), dtype=q.dtype, device=q.device)
-    to = torch.empty_like(o)
-    lse = torch.empty((B, H, Lq), dtype=torch.float32, device=q.device)
-    dlse = torch.empty_like(lse) if need_dlse else None
+    o = _empty((B, Lq, H, D), q.dtype, q.device)
+    to = _empty((B, Lq, H, D), q.dtype, q.device)
+    lse = _empty((B, H, Lq), torch.float32, q.device)
+    dlse = _empty((B, H, Lq), torch.float32, q.device) if need_dlse else None
     with torch.cuda.device(q.device):
         rc = load().dmf_attn_fwd_jvp(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(),
@@ -118,8 +133,8 @@ def fwd(q, k, v, scale: float, need_lse: bool = True):
     q, k, v = map(_prep, (q, k, v))
     B, Lq, H, D = q.shape
     Lkv = k.shape[1]
-    o = torch.empty((B, Lq, H, D), dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, H, Lq), dtype=torch.float32, device=q.device) if need_lse else None
+    o = _empty((B, Lq, H, D), q.dtype, q.device)
+    lse = _empty((B, H, Lq), torch.float32, q.device) if need_lse else None
     with torch.cuda.device(q.device):
         rc = load().dmf_attn_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if need_lse else None,
@@ -132,13 +147,13 @@ def bwd(dout, q, k, v, o, lse, scale: float):
     """Backward on the primal output.  Returns (dq, dk, dv), contiguous."""
     _check_inputs(q, k, v, o, dout)
     dout, q, k, v, o = map(_prep, (dout, q, k, v, o))
-    lse = lse.contiguous()
+    lse = _raw(_raw(lse).contiguous())
     B, Lq, H, D = q.shape
     Lkv = k.shape[1]
-    dq = torch.empty((B, Lq, H, D), dtype=q.dtype, device=q.device)
-    dk = torch.empty((B, Lkv, H, D), dtype=q.dtype, device=q.device)
-    dv = torch.empty_like(dk)
-    delta = torch.empty((B, H, Lq), dtype=torch.float32, device=q.device)
+    dq = _empty((B, Lq, H, D), q.dtype, q.device)
+    dk = _empty((B, Lkv, H, D), q.dtype, q.device)
+    dv = _empty((B, Lkv, H, D), q.dtype, q.device)
+    delta = _empty((B, H, Lq), torch.float32, q.device)
     with torch.cuda.device(q.device):
         rc = load().dmf_attn_bwd(
             dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),

@@ -21,17 +21,8 @@ from __future__ import annotations
 
 import torch
 import torch.autograd.forward_ad as fwAD
-from torch._C import _functorch
 
 from . import _lib
-
-
-def _raw(t):
-    """Strip functorch wrappers: inside ``jvp`` the saved tensors and tangents
-    arrive wrapped at the transform level and have no storage of their own."""
-    while t is not None and _functorch.is_functorch_wrapped_tensor(t):
-        t = _functorch.get_unwrapped(t)
-    return t
 
 
 def _default_scale(q: torch.Tensor, softmax_scale):
@@ -84,8 +75,8 @@ class FlashAttnFunc(torch.autograd.Function):
         # second-order quantity, which the reference does not provide either.
         if gq is None and gk is None and gv is None:
             return None, None, None
-        q, k, v = (_raw(t) for t in ctx.saved_tensors[:3])
-        gq, gk, gv = _raw(gq), _raw(gk), _raw(gv)
+        # (saved tensors and tangents arrive functorch-wrapped here; _lib unwraps them)
+        q, k, v = ctx.saved_tensors[:3]
         gq = torch.zeros_like(q) if gq is None else gq
         gk = torch.zeros_like(k) if gk is None else gk
         gv = torch.zeros_like(v) if gv is None else gv
