@@ -13,6 +13,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <utility>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -27,6 +28,16 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
 namespace dmf {
+
+// Compile-time unrolled loop: f(std::integral_constant<int, 0>{}) ... f(<N-1>).
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -112,6 +123,61 @@ __device__ __forceinline__ ColOperand lds_col_operand(const T* tile, int r0, int
     r.v = u32x4{__float_as_uint(tile[row * STRIDE + col0 + c32]), 0u, 0u, 0u};
   }
   return r;
+}
+
+// bf16 column operands issued as raw instructions that the compiler does not
+// model as LDS accesses.  Rationale: in front of the ds_read_b64_tr_b16
+// *intrinsic* the compiler places a full `s_waitcnt vmcnt(0)` whenever an
+// HBM->LDS DMA load is in flight, which would serialise the tile prefetch with
+// the math.  lds_tr16_issue() starts the two transposed reads of one operand
+// (rows r..r+3 at byte offset OFF_LO, rows r+8..r+11 at OFF_HI, relative to the
+// lane address described at lds_col_operand); lds_tr16_wait() must be applied
+// to the results before they are used.  LDS operations complete in order, so
+// these untracked reads only ever make the compiler's own lgkmcnt waits more
+// conservative.
+struct TrPair { u32x2 lo, hi; };
+
+template <int OFF_LO, int OFF_HI>
+__device__ __forceinline__ TrPair lds_tr16_issue(uint32_t lane_addr) {
+  TrPair r;
+  asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+               : "=&v"(r.lo), "=&v"(r.hi)
+               : "v"(lane_addr), "n"(OFF_LO), "n"(OFF_HI));
+  return r;
+}
+// Wait until at most N LDS instructions issued after these operands are still
+// outstanding (N = number of reads issued since, for software pipelining).
+template <int N>
+__device__ __forceinline__ void lds_tr16_wait(TrPair& a) {
+  asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(a.lo), "+v"(a.hi) : [n] "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_tr16_wait(TrPair& a, TrPair& b) {
+  asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi) : [n] "n"(N));
+}
+// Row-operand chunk (16 bytes per lane) issued the same untracked way.
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_read128_issue(uint32_t lane_addr) {
+  u32x4 r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(lane_addr), "n"(OFF));
+  return r;
+}
+template <int N>
+__device__ __forceinline__ void lds_read128_wait(u32x4& a) {
+  asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(a) : [n] "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_read128_wait(u32x4& a, u32x4& b) {
+  asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(a), "+v"(b) : [n] "n"(N));
+}
+__device__ __forceinline__ ColOperand tr_operand(const TrPair& a) {
+  ColOperand r;
+  r.v = u32x4{a.lo[0], a.lo[1], a.hi[0], a.hi[1]};
+  return r;
+}
+// Byte address in LDS of a pointer into the work-group's shared memory.
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)LDS_PTR(const char, p);
 }
 
 // Matching B operand built from a lane's accumulator tile (already converted to

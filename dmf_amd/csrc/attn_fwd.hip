@@ -223,9 +223,17 @@ static int launch_fwd_d(const FwdParams& p, int BH, int D, hipStream_t stream) {
   }
 }
 
-int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream) {
+int launch_fwd_generic(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream) {
   if (bf16) return jvp ? launch_fwd_d<__bf16, true>(p, BH, D, stream) : launch_fwd_d<__bf16, false>(p, BH, D, stream);
   return jvp ? launch_fwd_d<float, true>(p, BH, D, stream) : launch_fwd_d<float, false>(p, BH, D, stream);
+}
+
+int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream) {
+  if (bf16) {
+    const int rc = launch_fwd_bf16_fast(p, BH, D, jvp, stream);
+    if (rc != 1) return rc;   // 1 = no tuned kernel for this shape
+  }
+  return launch_fwd_generic(p, BH, D, bf16, jvp, stream);
 }
 
 }  // namespace dmf

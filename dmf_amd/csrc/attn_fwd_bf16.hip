@@ -1,0 +1,348 @@
+// Tuned bf16 attention forward (+ JVP) for gfx950.
+//
+// Same math and register layout as the generic kernel in attn_fwd.hip
+// (transposed scores S^T = K Q^T, per-lane softmax state, P^T fed back as the
+// MFMA B operand, O^T / dO^T accumulators), restructured for throughput:
+//   * <= 256 VGPRs so two work-groups (8 waves) share a CU and one wave's
+//     softmax VALU work overlaps another wave's MFMAs;
+//   * K, V, dK, dV tiles of 32 keys go HBM -> LDS with global_load_lds_dwordx4
+//     (no staging registers), double-buffered, one barrier per tile;
+//   * Q and dQ are pre-multiplied by the softmax scale when loaded, so neither
+//     S nor dS needs a per-element scale;
+//   * lazy rescaling: the running maximum is only raised (and O, dO rescaled)
+//     when a score exceeds it by more than 2^kLazyLog2, otherwise the stale
+//     maximum is kept -- exact, because normalisation happens once at the end;
+//   * for head dims that are not a multiple of 32 the spare row D of the last
+//     O^T / dO^T tile is fed a column of ones (V) / zeros (dV), so the MFMAs
+//     deliver the row sums l = sum(P) and mu = sum(P*dS) for free.
+#include "attn_common.h"
+#include "attn_kernels.h"
+#include <algorithm>
+
+namespace dmf {
+
+constexpr float kLazyLog2 = 6.0f;
+
+template <int D>
+struct FastCfg {
+  static constexpr int VPR = D / 8, NCHUNK = (D + 15) / 16, NDT = (D + 31) / 32;
+  static constexpr int KP = Cfg<__bf16, D>::ROWV;                         // K/dK row pitch in 16-byte vectors (odd)
+  static constexpr int VP = NDT * 4 <= 4 ? 4 : (NDT * 4 <= 12 ? 12 : 20);  // V/dV pitch: 4 (mod 8) vectors => conflict-free transposed reads
+  static constexpr int KSTR = KP * 8, VSTR = VP * 8;                       // pitches in elements
+  static constexpr int BKV = 32;
+  static constexpr int KBYTES = BKV * KP * 16, VBYTES = BKV * VP * 16;
+  static constexpr bool PADROW = (D % 32) != 0;
+  static constexpr int PAD_IDX = 4 * ((D % 32) / 8) + (D % 4);             // accumulator element holding row D%32 ...
+  static constexpr int PAD_G = ((D % 32) % 8) / 4;                         // ... in the lanes of this half
+};
+
+// Issue the HBM -> LDS loads of one tensor tile (32 rows): wave w moves rows
+// 8w..8w+7.  LDS placement is lane-linear (base + lane*16), which with a
+// row-major padded tile means slot = row*PITCH + vector; lanes that fall on
+// padding vectors are switched off.  The source is a raw buffer resource that
+// covers exactly the Lkv rows of this (batch, head): `soffset` selects the
+// tile, and rows past the end read as zeros (hardware bounds check).
+template <int PITCH, int VPR>
+__device__ __forceinline__ void issue_tile_rows(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_bytes, uint32_t soffset,
+                                                char* lds_tile, int wave, int lane) {
+  constexpr int SLOTS = 8 * PITCH;
+#pragma unroll
+  for (int i = 0; i < (SLOTS + 63) / 64; ++i) {
+    const int slot = 64 * i + lane;
+    const int r = slot / PITCH, cv = slot % PITCH;
+    if (slot < SLOTS && cv < VPR) {
+      const uint32_t voff = (uint32_t)(8 * wave + r) * row_bytes + cv * 16;
+      char* dst = lds_tile + (8 * wave * PITCH + 64 * i) * 16;   // wave-uniform
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, voff, soffset, 0, 0);
+    }
+  }
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* base, uint32_t row_bytes, int nrows, int row_payload_bytes) {
+  // raw buffer, byte-granular bounds: [base, base + (nrows-1)*row_bytes + payload)
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (nrows - 1) * row_bytes + row_payload_bytes, 0x00020000);
+}
+
+template <int D, bool JVP>
+__global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p) {
+  using F = FastCfg<D>;
+  using T = __bf16;
+  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NDT = F::NDT, KP = F::KP, VP = F::VP;
+  constexpr int KSTR = F::KSTR, VSTR = F::VSTR, BKV = F::BKV;
+  constexpr int STAGE = (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES);
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  auto Kt = [&](int s) { return smem + s * STAGE; };
+  auto Vt = [&](int s) { return smem + s * STAGE + F::KBYTES; };
+  auto dKt = [&](int s) { return smem + s * STAGE + F::KBYTES + F::VBYTES; };
+  auto dVt = [&](int s) { return smem + s * STAGE + 2 * F::KBYTES + F::VBYTES; };
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, g = lane >> 5;
+
+  const uint32_t nqb = (p.Lq + 127) / 128;
+  const uint32_t wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = wg / nqb, qb = wg % nqb;
+  const int b = bh / p.H, h = bh % p.H;
+  const int q0 = qb * 128;
+  auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
+  const T* gk = reinterpret_cast<const T*>(p.k) + base(1);
+  const T* gv = reinterpret_cast<const T*>(p.v) + base(2);
+  const T* gtk = JVP ? reinterpret_cast<const T*>(p.tk) + base(4) : nullptr;
+  const T* gtv = JVP ? reinterpret_cast<const T*>(p.tv) + base(5) : nullptr;
+
+  // ---- padding of both stages: zeros, and the ones column of V
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    for (int i = tid; i < BKV * (KP - VPR); i += 256) {
+      const int off = ((i / (KP - VPR)) * KP + VPR + i % (KP - VPR)) * 16;
+      *reinterpret_cast<u32x4*>(Kt(s) + off) = u32x4{0, 0, 0, 0};
+      if constexpr (JVP) *reinterpret_cast<u32x4*>(dKt(s) + off) = u32x4{0, 0, 0, 0};
+    }
+    if constexpr (VP > VPR) {
+      for (int i = tid; i < BKV * (VP - VPR); i += 256) {
+        const int cv = VPR + i % (VP - VPR);
+        const int off = ((i / (VP - VPR)) * VP + cv) * 16;
+        const bool ones = F::PADROW && cv == VPR;          // element D of the row = 1.0 (bf16 0x3f80)
+        *reinterpret_cast<u32x4*>(Vt(s) + off) = u32x4{ones ? 0x3f80u : 0u, 0, 0, 0};
+        if constexpr (JVP) *reinterpret_cast<u32x4*>(dVt(s) + off) = u32x4{0, 0, 0, 0};
+      }
+    }
+  }
+
+  // ---- Q, dQ operand chunks, pre-multiplied by the softmax scale
+  u32x4 Qr[NCHUNK], dQr[JVP ? NCHUNK : 1];
+  {
+    const int qrow = q0 + wave * 32 + c32;
+    const bool ok = qrow < p.Lq;
+    const T* gq = reinterpret_cast<const T*>(p.q) + base(0) + (int64_t)qrow * p.st[0][1];
+    const T* gtq = JVP ? reinterpret_cast<const T*>(p.tq) + base(3) + (int64_t)qrow * p.st[3][1] : nullptr;
+    auto scaled = [&](u32x4 x) {
+      u32x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        y[e] = pack_bf16x2(__uint_as_float(x[e] << 16) * p.scale, __uint_as_float(x[e] & 0xffff0000u) * p.scale);
+      return y;
+    };
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int cv = 2 * c + g;
+      const bool in = ok && cv < VPR;
+      Qr[c] = in ? scaled(*reinterpret_cast<const u32x4*>(gq + cv * 8)) : u32x4{0, 0, 0, 0};
+      if constexpr (JVP) dQr[c] = in ? scaled(*reinterpret_cast<const u32x4*>(gtq + cv * 8)) : u32x4{0, 0, 0, 0};
+    }
+  }
+
+  f32x16 O[NDT], dO[JVP ? NDT : 1];
+#pragma unroll
+  for (int t = 0; t < NDT; ++t) {
+    O[t] = f32x16{0};
+    if constexpr (JVP) dO[t] = f32x16{0};
+  }
+  float m_run = -INFINITY, l_run = 0.f, mu_run = 0.f;   // log2-domain running max; VALU row sums only when !PADROW
+
+  // Lane address for the transposed V / dV operand reads (see lds_col_operand):
+  // 16 lanes fetch a 4-row x 16-column block, lane i supplying row i/4, columns 4*(i%4)..+3.
+  constexpr int DV_OFF = F::KBYTES + F::VBYTES;   // dV tile sits this many bytes after the V tile
+  const uint32_t k_lane_addr = lds_addr(smem) + c32 * KSTR * 2 + g * 16;   // row-operand reads of K / dK
+  const uint32_t v_lane_addr =
+      lds_addr(smem) + F::KBYTES + ((4 * g + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  const uint32_t rb_k = (uint32_t)p.st[1][1] * 2, rb_v = (uint32_t)p.st[2][1] * 2;
+  const uint32_t rb_tk = JVP ? (uint32_t)p.st[4][1] * 2 : 0, rb_tv = JVP ? (uint32_t)p.st[5][1] * 2 : 0;
+  const __amdgpu_buffer_rsrc_t rs_k = make_rows_rsrc(gk, rb_k, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_v = make_rows_rsrc(gv, rb_v, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_tk = make_rows_rsrc(JVP ? gtk : gk, JVP ? rb_tk : rb_k, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_tv = make_rows_rsrc(JVP ? gtv : gv, JVP ? rb_tv : rb_v, p.Lkv, D * 2);
+  auto issue = [&](int it) {
+    const int s = it & 1;
+    const uint32_t r0 = (uint32_t)it * BKV;
+    issue_tile_rows<KP, VPR>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
+    issue_tile_rows<VP, VPR>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
+    if constexpr (JVP) {
+      issue_tile_rows<KP, VPR>(rs_tk, rb_tk, r0 * rb_tk, dKt(s), wave, lane);
+      issue_tile_rows<VP, VPR>(rs_tv, rb_tv, r0 * rb_tv, dVt(s), wave, lane);
+    }
+  };
+
+  const int ntiles = (p.Lkv + BKV - 1) / BKV;
+  issue(0);
+  for (int it = 0; it < ntiles; ++it) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile `it` has landed in LDS
+#ifndef DMF_EXP_NOBARRIER
+    __syncthreads();                       // ... and everyone else's; also: all waves are done with the other stage
+#endif
+#ifndef DMF_EXP_NOLOAD
+    if (it + 1 < ntiles) issue(it + 1);
+#endif
+    const int s = it & 1;
+
+    // ---- S^T (already scaled) and dS^T; the LDS reads of chunk c+1 are in
+    //      flight while the MFMAs of chunk c run
+    f32x16 S = {0}, dS = {0};
+    {
+      const uint32_t ka = k_lane_addr + s * STAGE;
+      u32x4 kc[2], dkc[2];
+      kc[0] = lds_read128_issue<0>(ka);
+      if constexpr (JVP) dkc[0] = lds_read128_issue<DV_OFF>(ka);
+      static_for<NCHUNK>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        constexpr bool more = c + 1 < NCHUNK;
+        if constexpr (more) {
+          kc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ka);
+          if constexpr (JVP) dkc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DV_OFF>(ka);
+        }
+        if constexpr (JVP) {
+          lds_read128_wait<more ? 2 : 0>(kc[c & 1], dkc[c & 1]);
+          mma_chunk<T>(S, kc[c & 1], Qr[c]);
+          mma_chunk<T>(dS, kc[c & 1], dQr[c]);
+          mma_chunk<T>(dS, dkc[c & 1], Qr[c]);
+        } else {
+          lds_read128_wait<more ? 1 : 0>(kc[c & 1]);
+          mma_chunk<T>(S, kc[c & 1], Qr[c]);
+        }
+      });
+    }
+    // ---- keys past the end (last tile only): their K/V rows were zero-filled, mask the scores
+    if ((it + 1) * BKV > p.Lkv) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (it * BKV + acc_row(i, g) >= p.Lkv) S[i] = -INFINITY;
+    }
+    // ---- lazy running maximum
+#ifdef DMF_EXP_NOSOFTMAX
+    f32x16 E = S, G = dS;
+#else
+    float mx = fmaxf(S[0], S[1]);
+#pragma unroll
+    for (int i = 2; i < 16; ++i) mx = fmaxf(mx, S[i]);
+    mx = xhalf_max(mx) * kLog2e;
+    if (__builtin_amdgcn_ballot_w64(mx > m_run + kLazyLog2) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2(m_run - m_new);
+      m_run = m_new;
+      if constexpr (!F::PADROW) {
+        l_run *= alpha;
+        if constexpr (JVP) mu_run *= alpha;
+      }
+#pragma unroll
+      for (int t = 0; t < NDT; ++t) {
+        O[t] *= alpha;
+        if constexpr (JVP) dO[t] *= alpha;
+      }
+    }
+    // ---- E = exp2(S log2e - m), G = E * dS
+    f32x16 E, G;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      E[i] = fast_exp2(fmaf(S[i], kLog2e, -m_run));
+      if constexpr (JVP) G[i] = E[i] * dS[i];
+      if constexpr (!F::PADROW) {
+        l_run += E[i];
+        if constexpr (JVP) mu_run += G[i];
+      }
+    }
+#endif
+    // ---- O^T += V^T P^T ; dO^T += V^T G^T + dV^T P^T, over 2*NDT operand groups
+    //      (step st, head-dim tile t); group i+1 is read while group i multiplies
+    {
+      const uint32_t va = v_lane_addr + s * STAGE;   // this lane's transposed-read address in the stage's V tile
+      ColOperand pe[2], pg[2];
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        pe[st] = acc_operand<T>(E, st);
+        if constexpr (JVP) pg[st] = acc_operand<T>(G, st);
+      }
+      constexpr int NG = 2 * NDT;
+      TrPair v[2], dv[2];
+      auto lo_off = [](int gi) constexpr { return (16 * (gi / NDT) * VSTR + 32 * (gi % NDT)) * 2; };
+      v[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * VSTR * 2>(va);
+      if constexpr (JVP) dv[0] = lds_tr16_issue<lo_off(0) + DV_OFF, lo_off(0) + 8 * VSTR * 2 + DV_OFF>(va);
+      static_for<NG>([&](auto gc) {
+        constexpr int gi = decltype(gc)::value;
+        constexpr int st = gi / NDT, t = gi % NDT;
+        constexpr bool more = gi + 1 < NG;
+        if constexpr (more) {
+          constexpr int LO = lo_off(gi + 1), HI = LO + 8 * VSTR * 2;
+          v[(gi + 1) & 1] = lds_tr16_issue<LO, HI>(va);
+          if constexpr (JVP) dv[(gi + 1) & 1] = lds_tr16_issue<LO + DV_OFF, HI + DV_OFF>(va);
+        }
+        if constexpr (JVP) {
+          lds_tr16_wait<more ? 4 : 0>(v[gi & 1], dv[gi & 1]);
+          mma_col<T>(O[t], tr_operand(v[gi & 1]), pe[st]);
+          mma_col<T>(dO[t], tr_operand(v[gi & 1]), pg[st]);
+          mma_col<T>(dO[t], tr_operand(dv[gi & 1]), pe[st]);
+        } else {
+          lds_tr16_wait<more ? 2 : 0>(v[gi & 1]);
+          mma_col<T>(O[t], tr_operand(v[gi & 1]), pe[st]);
+        }
+      });
+    }
+  }
+
+  // ---- epilogue
+  float l_tot, mu_tot = 0.f;
+  if constexpr (F::PADROW) {
+    auto pick = [&](float x) {
+      auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+      return __uint_as_float(r[F::PAD_G]);
+    };
+    l_tot = pick(O[NDT - 1][F::PAD_IDX]);
+    if constexpr (JVP) mu_tot = pick(dO[NDT - 1][F::PAD_IDX]);
+  } else {
+    l_tot = xhalf_sum(l_run);
+    if constexpr (JVP) mu_tot = xhalf_sum(mu_run);
+  }
+  const float inv_l = 1.0f / l_tot;
+  const float mu_n = mu_tot * inv_l;
+  {
+    const int qrow = q0 + wave * 32 + c32;
+    if (g == 0 && qrow < p.Lq) {
+      if (p.lse != nullptr) p.lse[(int64_t)bh * p.Lq + qrow] = (m_run + log2f(l_tot)) * kLn2;
+      if constexpr (JVP)
+        if (p.dlse != nullptr) p.dlse[(int64_t)bh * p.Lq + qrow] = mu_n;
+    }
+  }
+  T* stage = reinterpret_cast<T*>(smem);
+  store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.o) + base(6), p.st[6][1], q0, p.Lq, tid,
+                              [&](int t, int i) { return O[t][i] * inv_l; });
+  if constexpr (JVP)
+    store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.to) + base(7), p.st[7][1], q0, p.Lq, tid,
+                                [&](int t, int i) { return fmaf(-mu_n, O[t][i] * inv_l, dO[t][i] * inv_l); });
+}
+
+template <int D, bool JVP>
+static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
+  using F = FastCfg<D>;
+  constexpr int tiles = 2 * (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES) + 512;
+  constexpr int stage = 128 * Cfg<__bf16, D>::OROWV * 16;
+  constexpr int smem = tiles > stage ? tiles : stage;
+  auto kern = attn_fwd_bf16_kernel<D, JVP>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
+      return -7;
+    attr_set = true;
+  }
+  const uint32_t nqb = (p.Lq + 127) / 128;
+  hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+// Returns 1 if this translation unit has no kernel for the case (caller falls
+// back to the generic kernel), else 0 / negative error code.
+int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_t stream) {
+  // 32-bit buffer addressing: every (batch, head) slab of K/V rows must span < 2 GiB
+  const int64_t max_row = std::max(std::max(p.st[1][1], p.st[2][1]), jvp ? std::max(p.st[4][1], p.st[5][1]) : (int64_t)0);
+  if (max_row * 2 * (int64_t)(p.Lkv + 32) >= (int64_t)1 << 31) return 1;
+  switch (D) {
+    case 64: return jvp ? launch_fast_t<64, true>(p, BH, stream) : launch_fast_t<64, false>(p, BH, stream);
+    case 72: return jvp ? launch_fast_t<72, true>(p, BH, stream) : launch_fast_t<72, false>(p, BH, stream);
+    case 96: return jvp ? launch_fast_t<96, true>(p, BH, stream) : launch_fast_t<96, false>(p, BH, stream);
+    case 128: return jvp ? launch_fast_t<128, true>(p, BH, stream) : launch_fast_t<128, false>(p, BH, stream);
+    default: return 1;
+  }
+}
+
+}  // namespace dmf

@@ -30,6 +30,10 @@ struct BwdParams {
 
 // Return 0 or a negative DMF_ATTN_E* code.
 int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream);
+// Building blocks of launch_fwd: the generic kernels (fp32 and bf16, any length)
+// and the tuned bf16 kernels (returns 1 when it has no kernel for the case).
+int launch_fwd_generic(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream);
+int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_t stream);
 int launch_bwd(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream);
 
 }  // namespace dmf
