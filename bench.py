@@ -141,8 +141,8 @@ def cpu_baseline_config1():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="xl2_512px", choices=list(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
@@ -195,7 +195,7 @@ def main():
             for kind, fn in (("fwd_jvp", lambda: _lib.fwd_jvp(qw, kw, vw, tqw, tkw, tvw, scale)),
                              ("fwd", lambda: _lib.fwd(qw, kw, vw, scale)),
                              ("bwd", lambda: _lib.bwd(dow, qw, kw, vw, ow, lsew, scale))):
-                t_ms, _ = time_gpu(fn, max(10, args.steps // 2), 5)
+                t_ms, _ = time_gpu(fn, max(10, args.steps // 2), max(5, args.warmup // 2))
                 fl, by = attn_flops(Bw, Hw, Nw, Dw, kind), attn_bytes(Bw, Hw, Nw, Dw, kind)
                 row[kind] = {"ms": t_ms, "tflops": fl / t_ms / 1e9, "pct_bf16_mfma_peak": 100 * fl / t_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
                              "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS}

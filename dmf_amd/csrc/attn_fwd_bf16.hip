@@ -157,7 +157,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
   const __amdgpu_buffer_rsrc_t rs_tv = make_rows_rsrc(JVP ? gtv : gv, JVP ? rb_tv : rb_v, p.Lkv, D * 2);
   auto issue = [&](int it) {
     const int s = it & 1;
+#ifdef DMF_EXP_SAMETILE
+    const uint32_t r0 = 0;
+#else
     const uint32_t r0 = (uint32_t)it * BKV;
+#endif
     issue_tile_rows<KP, VPR>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
     issue_tile_rows<VP, VPR>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
     if constexpr (JVP) {

@@ -1,0 +1,140 @@
+"""DMFT harness model: the caller context of the attention operator.
+
+Host-side mirror of the reference's Decoupled MeanFlow Transformer
+(models/dmft.py:27-175): patch embedding + fixed sin-cos positions, ``dmf_depth``
+encoder blocks conditioned on (t, y), the remaining decoder blocks and the final
+layer conditioned on (r, y), optional log-variance head.  It exists so that the
+attention kernels can be exercised and timed exactly as the MeanFlow loss calls
+them (``torch.func.jvp`` through the whole model); ``attn_func`` selects the
+operator, ``"hip"`` being this package's kernels.
+"""
+from __future__ import annotations
+
+from functools import partial
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+from .layers import DiTBlock, FinalLayer, LabelEmbedder, TimestepEmbedder, get_2d_sincos_pos_embed, timestep_embedding
+
+
+class PatchEmbed(nn.Module):
+    """Image -> patch tokens with a strided convolution; same parameters and
+    output as the ``timm`` layer the reference uses (models/dmft.py:15,54-56):
+    ``proj = Conv2d(C_in, C, kernel=stride=patch)``, tokens in row-major order."""
+
+    def __init__(self, img_size: int, patch_size: int, in_chans: int, embed_dim: int, bias: bool = True):
+        super().__init__()
+        self.patch_size = patch_size
+        self.num_patches = (img_size // patch_size) ** 2
+        self.proj = nn.Conv2d(in_chans, embed_dim, kernel_size=patch_size, stride=patch_size, bias=bias)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.proj(x).flatten(2).transpose(1, 2)
+
+
+class DMFT(nn.Module):
+    """Reference models/dmft.py:27-151."""
+
+    def __init__(self, input_size: int = 32, patch_size: int = 2, in_channels: int = 4, hidden_size: int = 1152,
+                 depth: int = 28, num_heads: int = 16, mlp_ratio: float = 4.0, use_cfg_embedding: bool = True,
+                 num_classes: int = 1000, dmf_depth: int = 8, use_logvar: bool = False, **block_kwargs):
+        super().__init__()
+        self.input_size, self.patch_size = input_size, patch_size
+        self.in_channels = self.out_channels = in_channels
+        self.num_heads, self.num_classes = num_heads, num_classes
+        self.dmf_depth, self.use_logvar = dmf_depth, use_logvar
+
+        self.x_embedder = PatchEmbed(input_size, patch_size, in_channels, hidden_size, bias=True)
+        self.t_embedder = TimestepEmbedder(hidden_size)
+        self.y_embedder = LabelEmbedder(num_classes, hidden_size, use_cfg_embedding)
+        self.num_patches = self.x_embedder.num_patches
+        self.pos_embed = nn.Parameter(torch.zeros(1, self.num_patches, hidden_size), requires_grad=False)
+        self.blocks = nn.ModuleList(
+            [DiTBlock(hidden_size, num_heads, mlp_ratio=mlp_ratio, **block_kwargs) for _ in range(depth)])
+        self.final_layer = FinalLayer(hidden_size, patch_size, self.out_channels)
+        if use_logvar:
+            self.logvar_t_embedder = partial(timestep_embedding, dim=128)
+            self.logvar_linear = nn.Linear(256, 1)
+        self.initialize_weights()
+
+    def initialize_weights(self) -> None:
+        """The reference's initialisation (models/dmft.py:79-121): Xavier linears,
+        N(0, 0.02) embeddings, and zeroed adaLN gates / output layer -- which makes
+        every block an identity and the output zero at step 0."""
+        def _basic_init(m):
+            if isinstance(m, nn.Linear):
+                nn.init.xavier_uniform_(m.weight)
+                if m.bias is not None:
+                    nn.init.constant_(m.bias, 0)
+        self.apply(_basic_init)
+        pe = get_2d_sincos_pos_embed(self.pos_embed.shape[-1], int(self.num_patches ** 0.5))
+        self.pos_embed.data.copy_(torch.from_numpy(pe).float().unsqueeze(0))
+        w = self.x_embedder.proj.weight.data
+        nn.init.xavier_uniform_(w.view([w.shape[0], -1]))
+        nn.init.constant_(self.x_embedder.proj.bias, 0)
+        nn.init.normal_(self.y_embedder.embedding_table.weight, std=0.02)
+        nn.init.normal_(self.t_embedder.mlp[0].weight, std=0.02)
+        nn.init.normal_(self.t_embedder.mlp[2].weight, std=0.02)
+        for block in self.blocks:
+            nn.init.constant_(block.adaLN_modulation[-1].weight, 0)
+            nn.init.constant_(block.adaLN_modulation[-1].bias, 0)
+        nn.init.constant_(self.final_layer.adaLN_modulation[-1].weight, 0)
+        nn.init.constant_(self.final_layer.adaLN_modulation[-1].bias, 0)
+        nn.init.constant_(self.final_layer.linear.weight, 0)
+        nn.init.constant_(self.final_layer.linear.bias, 0)
+        if self.use_logvar:
+            nn.init.constant_(self.logvar_linear.weight, 0)
+            nn.init.constant_(self.logvar_linear.bias, 0)
+
+    def init_trunc_normal_(self, std: float = 0.02, seed: int = 0) -> "DMFT":
+        """Benchmark initialisation: every weight matrix / embedding ~ truncated
+        N(0, std) (cut at 2 std), biases zero.  With the reference's zero-gate
+        initialisation attention contributes nothing to the output, so timing and
+        parity runs use this instead."""
+        g = torch.Generator().manual_seed(seed)
+        for name, prm in self.named_parameters():
+            if name == "pos_embed":
+                continue
+            if prm.dim() >= 2:
+                w = torch.empty(prm.shape, dtype=torch.float32)
+                nn.init.trunc_normal_(w, std=std, a=-2 * std, b=2 * std, generator=g)
+                prm.data.copy_(w)
+            elif name.endswith("bias"):
+                prm.data.zero_()
+        return self
+
+    def unpatchify(self, x: Tensor) -> Tensor:
+        c, p = self.out_channels, self.patch_size
+        h = w = int(x.shape[1] ** 0.5)
+        assert h * w == x.shape[1]
+        x = x.reshape(x.shape[0], h, w, p, p, c)
+        x = torch.einsum("nhwpqc->nchpwq", x)
+        return x.reshape(x.shape[0], c, h * p, w * p)
+
+    def forward(self, x, t, r, y, return_logvar: bool = False):
+        t, r = t.reshape(-1), r.reshape(-1)
+        x = self.x_embedder(x) + self.pos_embed
+        B, L, D = x.shape
+        t_embed = self.t_embedder(t).reshape(B, -1, D)
+        y_embed = self.y_embedder(y).reshape(B, -1, D)
+        c_t = t_embed + y_embed
+        for block in self.blocks[:self.dmf_depth]:      # encoder: conditioned on t
+            x = block(x, c_t)
+        c_r = self.t_embedder(r).reshape(B, -1, D) + y_embed
+        for block in self.blocks[self.dmf_depth:]:      # decoder: conditioned on r
+            x = block(x, c_r)
+        x = self.unpatchify(self.final_layer(x, c_r))
+        if return_logvar:
+            logvar = self.logvar_linear(torch.cat([self.logvar_t_embedder(t), self.logvar_t_embedder(r)], dim=1))
+            return x, logvar.view(-1, *[1] * (x.ndim - 1))
+        return x
+
+
+# size registry (reference models/dmft.py:154-175)
+_SIZES = {"XL": (28, 1152, 16), "L": (24, 1024, 16), "M": (16, 1024, 16), "B": (12, 768, 12), "S": (12, 384, 6)}
+DMFT_models = {
+    f"DMFT-{s}/{p}": partial(DMFT, depth=d, hidden_size=h, patch_size=p, num_heads=nh)
+    for s, (d, h, nh) in _SIZES.items() for p in (2, 4, 8)
+}

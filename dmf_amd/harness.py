@@ -1,0 +1,99 @@
+"""MeanFlow JVP step and end-to-end timing of the DMFT harness.
+
+``meanflow_jvp`` restates the JVP call site of the reference's loss
+(loss.py:165-173): ``torch.func.jvp`` through the whole model with tangents
+(v, 1, 0) for (x_t, t, r), target ``u_tgt = v + (r - t) * du/dt`` detached.
+``train_step`` adds the backward on the primal output only, as
+train_dmf.py:325-330 does under bf16 autocast.
+"""
+from __future__ import annotations
+
+import time
+from functools import partial
+
+import torch
+
+from .dmft import DMFT_models
+
+
+def synthetic_batch(batch: int, device, seed: int = 2, input_size: int = 32, channels: int = 4, num_classes: int = 1000):
+    """z ~ N(0,1) (B,4,S,S); t, r ~ U(0,1) with r <= t, shaped (B,1,1,1) as the
+    reference's samplers produce them; labels uniform; tangent v ~ N(0,1)."""
+    g = torch.Generator().manual_seed(seed)
+    z = torch.randn(batch, channels, input_size, input_size, generator=g)
+    v = torch.randn(batch, channels, input_size, input_size, generator=g)
+    a, b = torch.rand(batch, 1, 1, 1, generator=g), torch.rand(batch, 1, 1, 1, generator=g)
+    t, r = torch.maximum(a, b), torch.minimum(a, b)
+    y = torch.randint(0, num_classes, (batch,), generator=g)
+    return tuple(x.to(device) for x in (z, t, r, y, v))
+
+
+def meanflow_jvp(model, x_t, t, r, y, v):
+    """(u, du_dt) = jvp(model(., ., ., y), (x_t, t, r), (v, 1, 0)) -- loss.py:165-170."""
+    model_fn = partial(model, y=y)
+    return torch.func.jvp(model_fn, (x_t, t, r), (v, torch.ones_like(t), torch.zeros_like(r)))
+
+
+def meanflow_loss(model, x_t, t, r, y, v):
+    """MeanFlow regression loss with the JVP target detached (loss.py:171-172);
+    plain mean-squared error (the log-variance weighting is not part of the path)."""
+    u, du_dt = meanflow_jvp(model, x_t, t, r, y, v)
+    u_tgt = (v + (r - t) * du_dt).detach()
+    return ((u - u_tgt) ** 2).mean(), u, du_dt
+
+
+def train_step(model, batch, autocast: bool = True):
+    """Forward + JVP, then backward on the primal output only."""
+    x_t, t, r, y, v = batch
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        loss, _, _ = meanflow_loss(model, x_t, t, r, y, v)
+    loss.backward()
+    return loss
+
+
+def build_model(name: str, attn_func: str, device, qk_norm: bool = False, input_size: int = 32, dmf_depth=None, seed: int = 0):
+    kw = {"attn_func": attn_func, "qk_norm": qk_norm, "input_size": input_size}
+    if dmf_depth is not None:
+        kw["dmf_depth"] = dmf_depth
+    return DMFT_models[name](**kw).init_trunc_normal_(0.02, seed).to(device)
+
+
+def _time(fn, steps: int, warmup: int = 2) -> float:
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True) -> dict:
+    """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast, and
+    (b) DMFT-XL/2 256px forward+JVP+backward, batch 32 -- each with the 'hip'
+    operator and, for reference, with the naive 'base' operator."""
+    out = {}
+    cases = [("DMFT-B/2", 64, 8, False), ("DMFT-XL/2", 32, 20, True)]
+    for name, batch, dmf_depth, train in cases:
+        row = {"batch": batch, "mode": "fwd+jvp+bwd" if train else "fwd+jvp", "dtype": "bf16 autocast"}
+        data = synthetic_batch(batch, device)
+        for op in (("hip", "base") if compare_base else ("hip",)):
+            model = build_model(name, op, device, dmf_depth=dmf_depth)
+            if train:
+                def fn():
+                    model.zero_grad(set_to_none=True)
+                    train_step(model, data)
+            else:
+                model.requires_grad_(False)
+
+                def fn():
+                    with torch.autocast("cuda", dtype=torch.bfloat16):
+                        meanflow_jvp(model, *data)
+            sec = _time(fn, steps if op == "hip" else max(2, steps // 2))
+            row[f"{op}_ms_per_step"] = sec * 1e3
+            row[f"{op}_images_per_s"] = batch / sec
+            del model
+            torch.cuda.empty_cache()
+        out[name] = row
+    return out
