@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdmf_attn.so")
-SOURCES = ["attn_fwd.hip", "attn_fwd_bf16.hip", "attn_bwd.hip", "dmf_attn_abi.hip"]
+SOURCES = ["attn_fwd.hip", "attn_fwd_bf16.hip", "attn_bwd.hip", "attn_bwd_bf16.hip", "dmf_attn_abi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

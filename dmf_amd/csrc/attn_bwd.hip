@@ -278,8 +278,16 @@ static int launch_bwd_d(const BwdParams& p, int BH, int D, hipStream_t stream) {
   }
 }
 
-int launch_bwd(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream) {
+int launch_bwd_generic(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream) {
   return bf16 ? launch_bwd_d<__bf16>(p, BH, D, stream) : launch_bwd_d<float>(p, BH, D, stream);
+}
+
+int launch_bwd(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream) {
+  if (bf16) {
+    const int rc = launch_bwd_bf16_fast(p, BH, D, stream);
+    if (rc != 1) return rc;   // 1 = no tuned kernel for this shape
+  }
+  return launch_bwd_generic(p, BH, D, bf16, stream);
 }
 
 }  // namespace dmf

@@ -1,0 +1,336 @@
+// Tuned bf16 backward (dQ kernel + dK/dV kernel) for gfx950.
+//
+// Same two-kernel, atomics-free scheme and the same register layouts as the
+// generic kernels in attn_bwd.hip, with the throughput structure of the tuned
+// forward: <= 256 VGPRs (two work-groups per CU), 32-row tiles streamed
+// HBM -> LDS by bounds-checked buffer DMA into a double buffer with one barrier
+// per tile, software-pipelined LDS operand reads, and the softmax scale and
+// log2(e) folded into the register-resident operand (Q in the dQ kernel, K in
+// the dK/dV kernel) so that P = exp2(S - lse*log2e) costs one VALU op + exp.
+#include "attn_common.h"
+#include "attn_kernels.h"
+#include <algorithm>
+
+namespace dmf {
+
+template <int D>
+struct BwdFastCfg {
+  static constexpr int VPR = D / 8, NCHUNK = (D + 15) / 16, NDT = (D + 31) / 32;
+  static constexpr int P = Cfg<__bf16, D>::ROWV;     // tile row pitch in 16-byte vectors (odd): tiles are read both by rows and transposed
+  static constexpr int STR = P * 8;
+  static constexpr int TBYTES = 32 * P * 16;          // one 32-row tile
+  static constexpr int STAT = 256;                    // per stage: 32 x lse, 32 x delta (fp32)
+};
+
+// bf16x8 chunk times a scalar, re-rounded to bf16.
+__device__ __forceinline__ u32x4 scale_bf16x8(u32x4 x, float s) {
+  u32x4 y;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    y[e] = pack_bf16x2(__uint_as_float(x[e] << 16) * s, __uint_as_float(x[e] & 0xffff0000u) * s);
+  return y;
+}
+
+template <int BYTES_PER_STAGE, int PADV, int P, int VPR>
+__device__ __forceinline__ void zero_pads(char* smem, int tile_off, int tid) {
+  if constexpr (PADV > 0) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+      for (int i = tid; i < 32 * PADV; i += 256)
+        *reinterpret_cast<u32x4*>(smem + s * BYTES_PER_STAGE + tile_off + ((i / PADV) * P + VPR + i % PADV) * 16) = u32x4{0, 0, 0, 0};
+  }
+}
+
+// ------------------------------------------------------------------ dQ kernel
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParams p) {
+  using F = BwdFastCfg<D>;
+  using T = __bf16;
+  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NDT = F::NDT, P = F::P, STR = F::STR;
+  constexpr int STAGE = 2 * F::TBYTES;   // K | V
+  constexpr int V_OFF = F::TBYTES;
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, g = lane >> 5;
+  const uint32_t nqb = (p.Lq + 127) / 128;
+  const uint32_t wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = wg / nqb, qb = wg % nqb;
+  const int b = bh / p.H, h = bh % p.H;
+  const int q0 = qb * 128;
+  auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
+
+  zero_pads<STAGE, P - VPR, P, VPR>(smem, 0, tid);
+  zero_pads<STAGE, P - VPR, P, VPR>(smem, V_OFF, tid);
+
+  // ---- this lane's query row: Q (times scale*log2e), dout, delta, lse
+  const int qrow = q0 + wave * 32 + c32;
+  const bool qok = qrow < p.Lq;
+  u32x4 Qr[NCHUNK], dOr[NCHUNK];
+  float dpart = 0.f;
+  {
+    const T* gq = reinterpret_cast<const T*>(p.q) + base(1) + (int64_t)qrow * p.st[1][1];
+    const T* gdo = reinterpret_cast<const T*>(p.dout) + base(0) + (int64_t)qrow * p.st[0][1];
+    const T* go = reinterpret_cast<const T*>(p.o) + base(4) + (int64_t)qrow * p.st[4][1];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int cv = 2 * c + g;
+      const bool in = qok && cv < VPR;
+      Qr[c] = in ? scale_bf16x8(*reinterpret_cast<const u32x4*>(gq + cv * 8), p.scale_log2) : u32x4{0, 0, 0, 0};
+      dOr[c] = in ? *reinterpret_cast<const u32x4*>(gdo + cv * 8) : u32x4{0, 0, 0, 0};
+      const u32x4 ov = in ? *reinterpret_cast<const u32x4*>(go + cv * 8) : u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        dpart += __uint_as_float(dOr[c][e] << 16) * __uint_as_float(ov[e] << 16);
+        dpart += __uint_as_float(dOr[c][e] & 0xffff0000u) * __uint_as_float(ov[e] & 0xffff0000u);
+      }
+    }
+  }
+  const float delta = xhalf_sum(dpart);
+  float lse2 = INFINITY;   // +inf switches padded query rows off (P = 0)
+  if (qok) {
+    lse2 = p.lse[(int64_t)bh * p.Lq + qrow] * kLog2e;
+    if (g == 0) p.delta[(int64_t)bh * p.Lq + qrow] = delta;
+  }
+
+  f32x16 dQ[NDT];
+#pragma unroll
+  for (int t = 0; t < NDT; ++t) dQ[t] = f32x16{0};
+
+  const uint32_t rb_k = (uint32_t)p.st[2][1] * 2, rb_v = (uint32_t)p.st[3][1] * 2;
+  const __amdgpu_buffer_rsrc_t rs_k = make_rows_rsrc(reinterpret_cast<const T*>(p.k) + base(2), rb_k, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_v = make_rows_rsrc(reinterpret_cast<const T*>(p.v) + base(3), rb_v, p.Lkv, D * 2);
+  auto issue = [&](int it) {
+    char* st = smem + (it & 1) * STAGE;
+    issue_tile_rows<P, VPR>(rs_k, rb_k, (uint32_t)it * 32 * rb_k, st, wave, lane);
+    issue_tile_rows<P, VPR>(rs_v, rb_v, (uint32_t)it * 32 * rb_v, st + V_OFF, wave, lane);
+  };
+  const uint32_t row_addr = lds_addr(smem) + c32 * STR * 2 + g * 16;
+  const uint32_t col_addr = lds_addr(smem) + ((4 * g + ((lane & 15) >> 2)) * STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  const int ntiles = (p.Lkv + 31) / 32;
+  issue(0);
+  for (int it = 0; it < ntiles; ++it) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    __syncthreads();
+    if (it + 1 < ntiles) issue(it + 1);
+    const uint32_t ra = row_addr + (it & 1) * STAGE, ca = col_addr + (it & 1) * STAGE;
+
+    // ---- S^T = K Q^T (log2 units), dP^T = V dout^T
+    f32x16 S = {0}, dP = {0};
+    {
+      u32x4 kc[2], vc[2];
+      kc[0] = lds_read128_issue<0>(ra);
+      vc[0] = lds_read128_issue<V_OFF>(ra);
+      static_for<NCHUNK>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        constexpr bool more = c + 1 < NCHUNK;
+        if constexpr (more) {
+          kc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
+          vc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + V_OFF>(ra);
+        }
+        lds_read128_wait<more ? 2 : 0>(kc[c & 1], vc[c & 1]);
+        mma_chunk<T>(S, kc[c & 1], Qr[c]);
+        mma_chunk<T>(dP, vc[c & 1], dOr[c]);
+      });
+    }
+    // ---- dS^T = P^T * (dP^T - delta)
+    f32x16 dS;
+    const bool tail = (it + 1) * 32 > p.Lkv;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float pr = fast_exp2(S[i] - lse2);
+      if (tail && it * 32 + acc_row(i, g) >= p.Lkv) pr = 0.f;
+      dS[i] = pr * (dP[i] - delta);
+    }
+    // ---- dQ^T += K^T dS^T
+    {
+      ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
+      constexpr int NG = 2 * NDT;
+      TrPair kk[2];
+      auto lo_off = [](int gi) constexpr { return (16 * (gi / NDT) * STR + 32 * (gi % NDT)) * 2; };
+      kk[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
+      static_for<NG>([&](auto gc) {
+        constexpr int gi = decltype(gc)::value;
+        constexpr bool more = gi + 1 < NG;
+        if constexpr (more) kk[(gi + 1) & 1] = lds_tr16_issue<lo_off(gi + 1), lo_off(gi + 1) + 8 * STR * 2>(ca);
+        lds_tr16_wait<more ? 2 : 0>(kk[gi & 1]);
+        mma_col<T>(dQ[gi % NDT], tr_operand(kk[gi & 1]), ds[gi / NDT]);
+      });
+    }
+  }
+  store_rows_transposed<T, D>(reinterpret_cast<T*>(smem), reinterpret_cast<T*>(p.dq) + base(5), p.st[5][1], q0, p.Lq, tid,
+                              [&](int t, int i) { return dQ[t][i] * p.scale; });
+}
+
+// --------------------------------------------------------------- dK/dV kernel
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdParams p) {
+  using F = BwdFastCfg<D>;
+  using T = __bf16;
+  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NDT = F::NDT, P = F::P, STR = F::STR;
+  constexpr int STAGE = 2 * F::TBYTES + F::STAT;   // Q | dout | lse[32], delta[32]
+  constexpr int DO_OFF = F::TBYTES, STAT_OFF = 2 * F::TBYTES;
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, g = lane >> 5;
+  const uint32_t nkb = (p.Lkv + 127) / 128;
+  const uint32_t wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = wg / nkb, kb = wg % nkb;
+  const int b = bh / p.H, h = bh % p.H;
+  const int k0 = kb * 128;
+  auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
+
+  zero_pads<STAGE, P - VPR, P, VPR>(smem, 0, tid);
+  zero_pads<STAGE, P - VPR, P, VPR>(smem, DO_OFF, tid);
+
+  // ---- this lane's key row: K (times scale*log2e) and V stay in registers
+  u32x4 Kr[NCHUNK], Vr[NCHUNK];
+  {
+    const int krow = k0 + wave * 32 + c32;
+    const bool ok = krow < p.Lkv;
+    const T* gk = reinterpret_cast<const T*>(p.k) + base(2) + (int64_t)krow * p.st[2][1];
+    const T* gv = reinterpret_cast<const T*>(p.v) + base(3) + (int64_t)krow * p.st[3][1];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int cv = 2 * c + g;
+      const bool in = ok && cv < VPR;
+      Kr[c] = in ? scale_bf16x8(*reinterpret_cast<const u32x4*>(gk + cv * 8), p.scale_log2) : u32x4{0, 0, 0, 0};
+      Vr[c] = in ? *reinterpret_cast<const u32x4*>(gv + cv * 8) : u32x4{0, 0, 0, 0};
+    }
+  }
+  f32x16 dK[NDT], dV[NDT];
+#pragma unroll
+  for (int t = 0; t < NDT; ++t) {
+    dK[t] = f32x16{0};
+    dV[t] = f32x16{0};
+  }
+
+  const uint32_t rb_q = (uint32_t)p.st[1][1] * 2, rb_do = (uint32_t)p.st[0][1] * 2;
+  const __amdgpu_buffer_rsrc_t rs_q = make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(1), rb_q, p.Lq, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_do = make_rows_rsrc(reinterpret_cast<const T*>(p.dout) + base(0), rb_do, p.Lq, D * 2);
+  // per-row statistics: padded query rows read lse = delta = 0; their Q and dout rows are zero, so they add nothing
+  const __amdgpu_buffer_rsrc_t rs_lse = make_rows_rsrc(p.lse + (int64_t)bh * p.Lq, 4, p.Lq, 4);
+  const __amdgpu_buffer_rsrc_t rs_dl = make_rows_rsrc(p.delta + (int64_t)bh * p.Lq, 4, p.Lq, 4);
+  auto issue = [&](int it) {
+    char* st = smem + (it & 1) * STAGE;
+    issue_tile_rows<P, VPR>(rs_q, rb_q, (uint32_t)it * 32 * rb_q, st, wave, lane);
+    issue_tile_rows<P, VPR>(rs_do, rb_do, (uint32_t)it * 32 * rb_do, st + DO_OFF, wave, lane);
+    if (wave < 2 && lane < 32)   // wave 0: lse[32], wave 1: delta[32]
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(wave == 0 ? rs_lse : rs_dl,
+                                               (__attribute__((address_space(3))) void*)(st + STAT_OFF + wave * 128), 4,
+                                               lane * 4, (uint32_t)it * 128, 0, 0);
+  };
+  const uint32_t row_addr = lds_addr(smem) + c32 * STR * 2 + g * 16;
+  const uint32_t col_addr = lds_addr(smem) + ((4 * g + ((lane & 15) >> 2)) * STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  const int ntiles = (p.Lq + 31) / 32;
+  issue(0);
+  for (int it = 0; it < ntiles; ++it) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    __syncthreads();
+    if (it + 1 < ntiles) issue(it + 1);
+    const uint32_t ra = row_addr + (it & 1) * STAGE, ca = col_addr + (it & 1) * STAGE;
+    const float* stat = reinterpret_cast<const float*>(smem + (it & 1) * STAGE + STAT_OFF);
+
+    // ---- S = Q K^T (log2 units), dP = dout V^T : rows = queries (in-lane), columns = keys (lanes)
+    f32x16 S = {0}, dP = {0};
+    {
+      u32x4 qc[2], oc[2];
+      qc[0] = lds_read128_issue<0>(ra);
+      oc[0] = lds_read128_issue<DO_OFF>(ra);
+      static_for<NCHUNK>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        constexpr bool more = c + 1 < NCHUNK;
+        if constexpr (more) {
+          qc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
+          oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
+        }
+        lds_read128_wait<more ? 2 : 0>(qc[c & 1], oc[c & 1]);
+        mma_chunk<T>(S, qc[c & 1], Kr[c]);
+        mma_chunk<T>(dP, oc[c & 1], Vr[c]);
+      });
+    }
+    // ---- P = exp2(S - lse*log2e), dS = P * (dP - delta)
+    f32x16 Pm, dS;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(stat + j * 8 + 4 * g);
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(stat + 32 + j * 8 + 4 * g);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = 4 * j + e;
+        Pm[i] = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
+        dS[i] = Pm[i] * (dP[i] - d4[e]);
+      }
+    }
+    // ---- dV^T += dout^T P ; dK^T += Q^T dS
+    {
+      ColOperand pp[2] = {acc_operand<T>(Pm, 0), acc_operand<T>(Pm, 1)};
+      ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
+      constexpr int NG = 2 * NDT;
+      TrPair qq[2], oo[2];
+      auto lo_off = [](int gi) constexpr { return (16 * (gi / NDT) * STR + 32 * (gi % NDT)) * 2; };
+      qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
+      oo[0] = lds_tr16_issue<lo_off(0) + DO_OFF, lo_off(0) + 8 * STR * 2 + DO_OFF>(ca);
+      static_for<NG>([&](auto gc) {
+        constexpr int gi = decltype(gc)::value;
+        constexpr bool more = gi + 1 < NG;
+        if constexpr (more) {
+          constexpr int LO = lo_off(gi + 1), HI = LO + 8 * STR * 2;
+          qq[(gi + 1) & 1] = lds_tr16_issue<LO, HI>(ca);
+          oo[(gi + 1) & 1] = lds_tr16_issue<LO + DO_OFF, HI + DO_OFF>(ca);
+        }
+        lds_tr16_wait<more ? 4 : 0>(qq[gi & 1], oo[gi & 1]);
+        mma_col<T>(dV[gi % NDT], tr_operand(oo[gi & 1]), pp[gi / NDT]);
+        mma_col<T>(dK[gi % NDT], tr_operand(qq[gi & 1]), ds[gi / NDT]);
+      });
+    }
+  }
+  T* stage = reinterpret_cast<T*>(smem);
+  store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.dk) + base(6), p.st[6][1], k0, p.Lkv, tid,
+                              [&](int t, int i) { return dK[t][i] * p.scale; });
+  store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.dv) + base(7), p.st[7][1], k0, p.Lkv, tid,
+                              [&](int t, int i) { return dV[t][i]; });
+}
+
+template <int D>
+static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
+  using F = BwdFastCfg<D>;
+  constexpr int tiles = 2 * (2 * F::TBYTES + F::STAT) + 512;
+  constexpr int stage = 128 * Cfg<__bf16, D>::OROWV * 16;
+  constexpr int smem = tiles > stage ? tiles : stage;
+  auto k1 = attn_bwd_dq_bf16_kernel<D>;
+  auto k2 = attn_bwd_dkv_bf16_kernel<D>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
+      return -7;
+    attr_set = true;
+  }
+  const uint32_t nqb = (p.Lq + 127) / 128, nkb = (p.Lkv + 127) / 128;
+  hipLaunchKernelGGL(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
+  if (hipGetLastError() != hipSuccess) return -7;
+  hipLaunchKernelGGL(k2, dim3(nkb * (uint32_t)BH), dim3(256), smem, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+// Returns 1 if there is no tuned kernel for the case (caller uses the generic ones).
+int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream) {
+  // 32-bit buffer addressing: every (batch, head) slab of rows must span < 2 GiB
+  const int64_t max_row = std::max(std::max(p.st[0][1], p.st[1][1]), std::max(p.st[2][1], p.st[3][1]));
+  if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 32) >= (int64_t)1 << 31) return 1;
+  switch (D) {
+    case 64: return launch_bwd_fast_t<64>(p, BH, stream);
+    case 72: return launch_bwd_fast_t<72>(p, BH, stream);
+    case 96: return launch_bwd_fast_t<96>(p, BH, stream);
+    case 128: return launch_bwd_fast_t<128>(p, BH, stream);
+    default: return 1;
+  }
+}
+
+}  // namespace dmf

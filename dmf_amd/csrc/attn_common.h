@@ -300,4 +300,31 @@ __device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t
   }
 }
 
+// Issue the HBM -> LDS loads of one tensor tile (32 rows): wave w moves rows
+// 8w..8w+7.  LDS placement is lane-linear (base + lane*16), which with a
+// row-major padded tile means slot = row*PITCH + vector; lanes that fall on
+// padding vectors are switched off.  The source is a raw buffer resource that
+// covers exactly the Lkv rows of this (batch, head): `soffset` selects the
+// tile, and rows past the end read as zeros (hardware bounds check).
+template <int PITCH, int VPR>
+__device__ __forceinline__ void issue_tile_rows(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_bytes, uint32_t soffset,
+                                                char* lds_tile, int wave, int lane) {
+  constexpr int SLOTS = 8 * PITCH;
+#pragma unroll
+  for (int i = 0; i < (SLOTS + 63) / 64; ++i) {
+    const int slot = 64 * i + lane;
+    const int r = slot / PITCH, cv = slot % PITCH;
+    if (slot < SLOTS && cv < VPR) {
+      const uint32_t voff = (uint32_t)(8 * wave + r) * row_bytes + cv * 16;
+      char* dst = lds_tile + (8 * wave * PITCH + 64 * i) * 16;   // wave-uniform
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, voff, soffset, 0, 0);
+    }
+  }
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* base, uint32_t row_bytes, int nrows, int row_payload_bytes) {
+  // raw buffer, byte-granular bounds: [base, base + (nrows-1)*row_bytes + payload)
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (nrows - 1) * row_bytes + row_payload_bytes, 0x00020000);
+}
+
 }  // namespace dmf

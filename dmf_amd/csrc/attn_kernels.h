@@ -34,6 +34,8 @@ int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream
 // and the tuned bf16 kernels (returns 1 when it has no kernel for the case).
 int launch_fwd_generic(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream);
 int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_t stream);
+int launch_bwd_generic(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream);
+int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream);
 int launch_bwd(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream);
 
 }  // namespace dmf
