@@ -30,6 +30,9 @@ if ROOT not in sys.path:
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the fused fwd+JVP kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (each scaled by what the counter reads for a plain 1 GiB copy; summary in profiles/attn_fwd_jvp_bf16_d72_xl2_512px.txt)
+MEASURED_TRAFFIC_BYTES = {"xl2_512px": 1.2768e9}
 
 WORKLOADS = {
     # name: (B, H, N, D, qk_norm)
@@ -185,7 +188,7 @@ def main():
                    "flops_per_step": flops, "hbm_bytes_per_step": attn_bytes(B, H, N, D, "fwd_jvp"),
                    "wall_ms_per_step": wall_ms},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "kernel": "dmf::attn_fwd_bf16_kernel<72, true>",
                      "hbm_gbs_algorithmic": attn_bytes(B, H, N, D, "fwd_jvp") / (ms * 1e-3) / 1e9},
     }
