@@ -175,6 +175,25 @@ __device__ __forceinline__ ColOperand tr_operand(const TrPair& a) {
   r.v = u32x4{a.lo[0], a.lo[1], a.hi[0], a.hi[1]};
   return r;
 }
+// 16x16x32 bf16 MFMA on the same operand containers (A/B: lane = index % 16,
+// contraction slots 8*(lane/16)..+7; C: column = lane % 16, rows 4*(lane/16)..+3).
+__device__ __forceinline__ void mma16(f32x4& acc, const ColOperand& a, const ColOperand& b) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a.v), __builtin_bit_cast(bf16x8, b.v), acc, 0, 0, 0);
+}
+// v_permlane16_swap: returns {x.row0, y.row0, x.row2, y.row2} and {x.row1, y.row1, x.row3, y.row3}
+// (rows = groups of 16 lanes).
+__device__ __forceinline__ void swap16(uint32_t x, uint32_t y, uint32_t& even, uint32_t& odd) {
+  auto r = __builtin_amdgcn_permlane16_swap(x, y, false, false);
+  even = r[0];
+  odd = r[1];
+}
+__device__ __forceinline__ void swap16f(float x, float& even, float& odd) {
+  uint32_t a, b;
+  swap16(__float_as_uint(x), __float_as_uint(x), a, b);
+  even = __uint_as_float(a);
+  odd = __uint_as_float(b);
+}
+
 // Byte address in LDS of a pointer into the work-group's shared memory.
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)LDS_PTR(const char, p);
@@ -278,21 +297,29 @@ __device__ __forceinline__ void zero_tile_padding(T* tile, int tid) {
 // Epilogue helper: a work-group's NDT transposed accumulator tiles (lane = output
 // row wave*32+c32, in-lane = head-dim index) are scaled, transposed through the
 // LDS staging area and stored with coalesced 16-byte rows.  Must be called by
-// all 256 threads; `stage` may alias the tile buffers (the leading barrier
+// all 64*NW threads of the work-group (NW waves, 32 rows each); `stage` may alias the tile buffers (the leading barrier
 // protects them).
-template <typename T, int D, typename F>
-__device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t row_stride, int row0, int nrows, int tid, F value) {
+//
+// NMAIN (default: all NDT tiles) limits `value` to the first NMAIN 32-wide tiles;
+// `tail(wave_stage)` may then write the remaining columns itself (wave_stage =
+// staging row 0 of this wave, row pitch Cfg::OSTRIDE).
+struct NoTail { __device__ __forceinline__ void operator()(void*) const {} };
+
+template <typename T, int D, int NW = 4, int NMAIN = Cfg<T, D>::NDT, typename F, typename TF = NoTail>
+__device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t row_stride, int row0, int nrows, int tid, F value,
+                                                      TF tail = TF{}) {
   using C = Cfg<T, D>;
   const int lane = tid & 63, wave = tid >> 6, c32 = lane & 31, g = lane >> 5;
   __syncthreads();
   T* srow = stage + (wave * 32 + c32) * C::OSTRIDE;
 #pragma unroll
-  for (int t = 0; t < C::NDT; ++t)
+  for (int t = 0; t < NMAIN; ++t)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       store4<T>(srow + t * 32 + j * 8 + 4 * g, value(t, 4 * j), value(t, 4 * j + 1), value(t, 4 * j + 2), value(t, 4 * j + 3));
+  tail(stage + wave * 32 * C::OSTRIDE);
   __syncthreads();
-  for (int v = tid; v < 128 * C::VPR; v += 256) {
+  for (int v = tid; v < 32 * NW * C::VPR; v += 64 * NW) {
     const int row = v / C::VPR, cv = v % C::VPR;
     if (row0 + row < nrows)
       *reinterpret_cast<u32x4*>(gdst + (int64_t)(row0 + row) * row_stride + cv * C::VEC) =
@@ -300,23 +327,24 @@ __device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t
   }
 }
 
-// Issue the HBM -> LDS loads of one tensor tile (32 rows): wave w moves rows
-// 8w..8w+7.  LDS placement is lane-linear (base + lane*16), which with a
+// Issue the HBM -> LDS loads of one tensor tile (32 rows): wave w of the NW waves
+// moves rows (32/NW)*w .. (32/NW)*(w+1)-1.  LDS placement is lane-linear (base + lane*16), which with a
 // row-major padded tile means slot = row*PITCH + vector; lanes that fall on
 // padding vectors are switched off.  The source is a raw buffer resource that
 // covers exactly the Lkv rows of this (batch, head): `soffset` selects the
 // tile, and rows past the end read as zeros (hardware bounds check).
-template <int PITCH, int VPR>
+template <int PITCH, int VPR, int NW = 4>
 __device__ __forceinline__ void issue_tile_rows(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_bytes, uint32_t soffset,
                                                 char* lds_tile, int wave, int lane) {
-  constexpr int SLOTS = 8 * PITCH;
+  constexpr int RPW = 32 / NW;          // rows per wave
+  constexpr int SLOTS = RPW * PITCH;
 #pragma unroll
   for (int i = 0; i < (SLOTS + 63) / 64; ++i) {
     const int slot = 64 * i + lane;
     const int r = slot / PITCH, cv = slot % PITCH;
     if (slot < SLOTS && cv < VPR) {
-      const uint32_t voff = (uint32_t)(8 * wave + r) * row_bytes + cv * 16;
-      char* dst = lds_tile + (8 * wave * PITCH + 64 * i) * 16;   // wave-uniform
+      const uint32_t voff = (uint32_t)(RPW * wave + r) * row_bytes + cv * 16;
+      char* dst = lds_tile + (RPW * wave * PITCH + 64 * i) * 16;   // wave-uniform
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, voff, soffset, 0, 0);
     }
   }

@@ -18,6 +18,7 @@
 #include "attn_common.h"
 #include "attn_kernels.h"
 #include <algorithm>
+#include <cstdlib>
 
 namespace dmf {
 
@@ -31,13 +32,23 @@ struct FastCfg {
   static constexpr int KSTR = KP * 8, VSTR = VP * 8;                       // pitches in elements
   static constexpr int BKV = 32;
   static constexpr int KBYTES = BKV * KP * 16, VBYTES = BKV * VP * 16;
-  static constexpr bool PADROW = (D % 32) != 0;
-  static constexpr int PAD_IDX = 4 * ((D % 32) / 8) + (D % 4);             // accumulator element holding row D%32 ...
+  // Head dims with a remainder of at most 16 over a multiple of 32 (72, 80): the
+  // remainder columns of O^T / dO^T are produced by 16x16x32 MFMAs instead of a
+  // mostly-padding 32-wide tile.
+  static constexpr bool TAIL = (D % 32) != 0 && (D % 32) <= 16;
+  static constexpr int NMT = TAIL ? D / 32 : NDT;                          // full 32-wide output tiles
+  // A spare output row (index D) exists when D is not a multiple of the tile width.
+  static constexpr bool PADROW = TAIL ? (D % 32) < 16 : (D % 32) != 0;
+  static constexpr int PAD_IDX = 4 * ((D % 32) / 8) + (D % 4);             // 32-wide last tile: accumulator element holding row D%32 ...
   static constexpr int PAD_G = ((D % 32) % 8) / 4;                         // ... in the lanes of this half
+  static constexpr int PAD16_ROW = (D % 32) / 4, PAD16_E = D % 4;          // 16-wide tail: lanes of 16-lane row PAD16_ROW, element PAD16_E
 };
 
-template <int D, bool JVP>
-__global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p) {
+// NW = waves per work-group: 4 (128 query rows, two work-groups per CU) or
+// 8 (256 query rows, one work-group per CU: half the tile traffic per FLOP).
+template <int D, bool JVP, int NW>
+__global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const FwdParams p) {
+  constexpr int NTHR = 64 * NW, BQ = 32 * NW;
   using F = FastCfg<D>;
   using T = __bf16;
   constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NDT = F::NDT, KP = F::KP, VP = F::VP;
@@ -54,11 +65,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, g = lane >> 5;
 
-  const uint32_t nqb = (p.Lq + 127) / 128;
+  const uint32_t nqb = (p.Lq + BQ - 1) / BQ;
   const uint32_t wg = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = wg / nqb, qb = wg % nqb;
   const int b = bh / p.H, h = bh % p.H;
-  const int q0 = qb * 128;
+  const int q0 = qb * BQ;
   auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
   const T* gk = reinterpret_cast<const T*>(p.k) + base(1);
   const T* gv = reinterpret_cast<const T*>(p.v) + base(2);
@@ -68,13 +79,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
   // ---- padding of both stages: zeros, and the ones column of V
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    for (int i = tid; i < BKV * (KP - VPR); i += 256) {
+    for (int i = tid; i < BKV * (KP - VPR); i += NTHR) {
       const int off = ((i / (KP - VPR)) * KP + VPR + i % (KP - VPR)) * 16;
       *reinterpret_cast<u32x4*>(Kt(s) + off) = u32x4{0, 0, 0, 0};
       if constexpr (JVP) *reinterpret_cast<u32x4*>(dKt(s) + off) = u32x4{0, 0, 0, 0};
     }
     if constexpr (VP > VPR) {
-      for (int i = tid; i < BKV * (VP - VPR); i += 256) {
+      for (int i = tid; i < BKV * (VP - VPR); i += NTHR) {
         const int cv = VPR + i % (VP - VPR);
         const int off = ((i / (VP - VPR)) * VP + cv) * 16;
         const bool ones = F::PADROW && cv == VPR;          // element D of the row = 1.0 (bf16 0x3f80)
@@ -107,11 +118,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
     }
   }
 
-  f32x16 O[NDT], dO[JVP ? NDT : 1];
+  constexpr int NMT = F::NMT;
+  constexpr bool TAIL = F::TAIL;
+  f32x16 O[NMT], dO[JVP ? NMT : 1];        // full 32-wide tiles of O^T / dO^T
+  f32x4 O16[2], dO16[2];                   // TAIL: 16-wide remainder, one 16x16 tile per half of the wave's 32 queries
 #pragma unroll
-  for (int t = 0; t < NDT; ++t) {
+  for (int t = 0; t < NMT; ++t) {
     O[t] = f32x16{0};
     if constexpr (JVP) dO[t] = f32x16{0};
+  }
+#pragma unroll
+  for (int hq = 0; hq < 2; ++hq) {
+    O16[hq] = f32x4{0, 0, 0, 0};
+    dO16[hq] = f32x4{0, 0, 0, 0};
   }
   float m_run = -INFINITY, l_run = 0.f, mu_run = 0.f;   // log2-domain running max; VALU row sums only when !PADROW
 
@@ -121,6 +140,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
   const uint32_t k_lane_addr = lds_addr(smem) + c32 * KSTR * 2 + g * 16;   // row-operand reads of K / dK
   const uint32_t v_lane_addr =
       lds_addr(smem) + F::KBYTES + ((4 * g + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  // Remainder (16x16x32) operand: 16-lane row w covers keys 16*(w%2) + 4*(w/2) + {0..3, 8..11} -- the keys whose
+  // probabilities that row receives from swap16 -- at head-dim columns 32*NMT .. 32*NMT+15.
+  const uint32_t t_lane_addr = lds_addr(smem) + F::KBYTES +
+      ((16 * ((lane >> 4) & 1) + 4 * (lane >> 5) + ((lane & 15) >> 2)) * VSTR + 32 * F::NMT + 4 * (lane & 3)) * 2;
 
   const uint32_t rb_k = (uint32_t)p.st[1][1] * 2, rb_v = (uint32_t)p.st[2][1] * 2;
   const uint32_t rb_tk = JVP ? (uint32_t)p.st[4][1] * 2 : 0, rb_tv = JVP ? (uint32_t)p.st[5][1] * 2 : 0;
@@ -135,11 +158,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
 #else
     const uint32_t r0 = (uint32_t)it * BKV;
 #endif
-    issue_tile_rows<KP, VPR>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
-    issue_tile_rows<VP, VPR>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
+    issue_tile_rows<KP, VPR, NW>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
+    issue_tile_rows<VP, VPR, NW>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
     if constexpr (JVP) {
-      issue_tile_rows<KP, VPR>(rs_tk, rb_tk, r0 * rb_tk, dKt(s), wave, lane);
-      issue_tile_rows<VP, VPR>(rs_tv, rb_tv, r0 * rb_tv, dVt(s), wave, lane);
+      issue_tile_rows<KP, VPR, NW>(rs_tk, rb_tk, r0 * rb_tk, dKt(s), wave, lane);
+      issue_tile_rows<VP, VPR, NW>(rs_tv, rb_tv, r0 * rb_tv, dVt(s), wave, lane);
     }
   };
 
@@ -204,9 +227,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
         if constexpr (JVP) mu_run *= alpha;
       }
 #pragma unroll
-      for (int t = 0; t < NDT; ++t) {
+      for (int t = 0; t < NMT; ++t) {
         O[t] *= alpha;
         if constexpr (JVP) dO[t] *= alpha;
+      }
+      if constexpr (TAIL) {
+        float a0, a1;   // alpha of query (lane % 16) and of query 16 + (lane % 16)
+        swap16f(alpha, a0, a1);
+        O16[0] *= a0;
+        O16[1] *= a1;
+        if constexpr (JVP) {
+          dO16[0] *= a0;
+          dO16[1] *= a1;
+        }
       }
     }
     // ---- E = exp2(S log2e - m), G = E * dS
@@ -221,8 +254,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
       }
     }
 #endif
-    // ---- O^T += V^T P^T ; dO^T += V^T G^T + dV^T P^T, over 2*NDT operand groups
-    //      (step st, head-dim tile t); group i+1 is read while group i multiplies
+    // ---- O^T += V^T P^T ; dO^T += V^T G^T + dV^T P^T, over 2*NMT operand groups
+    //      (step st, head-dim tile t) plus, with TAIL, one 16-wide remainder group;
+    //      group i+1 is read while group i multiplies
     {
       const uint32_t va = v_lane_addr + s * STAGE;   // this lane's transposed-read address in the stage's V tile
       ColOperand pe[2], pg[2];
@@ -231,28 +265,55 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
         pe[st] = acc_operand<T>(E, st);
         if constexpr (JVP) pg[st] = acc_operand<T>(G, st);
       }
-      constexpr int NG = 2 * NDT;
+      constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
       TrPair v[2], dv[2];
-      auto lo_off = [](int gi) constexpr { return (16 * (gi / NDT) * VSTR + 32 * (gi % NDT)) * 2; };
+      auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * VSTR + 32 * (gi % NMT)) * 2; };
       v[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * VSTR * 2>(va);
       if constexpr (JVP) dv[0] = lds_tr16_issue<lo_off(0) + DV_OFF, lo_off(0) + 8 * VSTR * 2 + DV_OFF>(va);
-      static_for<NG>([&](auto gc) {
+      static_for<NGT>([&](auto gc) {
         constexpr int gi = decltype(gc)::value;
-        constexpr int st = gi / NDT, t = gi % NDT;
-        constexpr bool more = gi + 1 < NG;
-        if constexpr (more) {
+        constexpr bool more = gi + 1 < NGT;
+        if constexpr (gi + 1 < NG) {
           constexpr int LO = lo_off(gi + 1), HI = LO + 8 * VSTR * 2;
           v[(gi + 1) & 1] = lds_tr16_issue<LO, HI>(va);
           if constexpr (JVP) dv[(gi + 1) & 1] = lds_tr16_issue<LO + DV_OFF, HI + DV_OFF>(va);
+        } else if constexpr (more) {   // the remainder group: all 32 keys in one 16x16x32 operand
+          const uint32_t ta = t_lane_addr + s * STAGE;
+          v[(gi + 1) & 1] = lds_tr16_issue<0, 8 * VSTR * 2>(ta);
+          if constexpr (JVP) dv[(gi + 1) & 1] = lds_tr16_issue<DV_OFF, 8 * VSTR * 2 + DV_OFF>(ta);
         }
-        if constexpr (JVP) {
-          lds_tr16_wait<more ? 4 : 0>(v[gi & 1], dv[gi & 1]);
+        if constexpr (JVP) lds_tr16_wait<more ? 4 : 0>(v[gi & 1], dv[gi & 1]);
+        else lds_tr16_wait<more ? 2 : 0>(v[gi & 1]);
+        if constexpr (gi < NG) {
+          constexpr int st = gi / NMT, t = gi % NMT;
           mma_col<T>(O[t], tr_operand(v[gi & 1]), pe[st]);
-          mma_col<T>(dO[t], tr_operand(v[gi & 1]), pg[st]);
-          mma_col<T>(dO[t], tr_operand(dv[gi & 1]), pe[st]);
+          if constexpr (JVP) {
+            mma_col<T>(dO[t], tr_operand(v[gi & 1]), pg[st]);
+            mma_col<T>(dO[t], tr_operand(dv[gi & 1]), pe[st]);
+          }
         } else {
-          lds_tr16_wait<more ? 2 : 0>(v[gi & 1]);
-          mma_col<T>(O[t], tr_operand(v[gi & 1]), pe[st]);
+          // B operands for the two query halves: lanes of 16-lane row w take (half g = w/2, step st = w%2)
+          ColOperand pe0, pe1, pg0, pg1;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            uint32_t ev, od;
+            swap16(pe[0].v[r], pe[1].v[r], ev, od);
+            pe0.v[r] = ev;
+            pe1.v[r] = od;
+            if constexpr (JVP) {
+              swap16(pg[0].v[r], pg[1].v[r], ev, od);
+              pg0.v[r] = ev;
+              pg1.v[r] = od;
+            }
+          }
+          mma16(O16[0], tr_operand(v[gi & 1]), pe0);
+          mma16(O16[1], tr_operand(v[gi & 1]), pe1);
+          if constexpr (JVP) {
+            mma16(dO16[0], tr_operand(v[gi & 1]), pg0);
+            mma16(dO16[1], tr_operand(v[gi & 1]), pg1);
+            mma16(dO16[0], tr_operand(dv[gi & 1]), pe0);
+            mma16(dO16[1], tr_operand(dv[gi & 1]), pe1);
+          }
         }
       });
     }
@@ -260,13 +321,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
 
   // ---- epilogue
   float l_tot, mu_tot = 0.f;
-  if constexpr (F::PADROW) {
+  if constexpr (F::PADROW && TAIL) {
+    // row D of the remainder tiles: 16-lane row PAD16_ROW holds it for query (lane % 16) [+16 in the second tile]
+    const int src = 16 * F::PAD16_ROW + (c32 & 15);
+    const float x0 = __shfl(O16[0][F::PAD16_E], src), x1 = __shfl(O16[1][F::PAD16_E], src);
+    l_tot = c32 < 16 ? x0 : x1;
+    if constexpr (JVP) {
+      const float y0 = __shfl(dO16[0][F::PAD16_E], src), y1 = __shfl(dO16[1][F::PAD16_E], src);
+      mu_tot = c32 < 16 ? y0 : y1;
+    }
+  } else if constexpr (F::PADROW) {
     auto pick = [&](float x) {
       auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
       return __uint_as_float(r[F::PAD_G]);
     };
-    l_tot = pick(O[NDT - 1][F::PAD_IDX]);
-    if constexpr (JVP) mu_tot = pick(dO[NDT - 1][F::PAD_IDX]);
+    l_tot = pick(O[NMT - 1][F::PAD_IDX]);
+    if constexpr (JVP) mu_tot = pick(dO[NMT - 1][F::PAD_IDX]);
   } else {
     l_tot = xhalf_sum(l_run);
     if constexpr (JVP) mu_tot = xhalf_sum(mu_run);
@@ -282,29 +352,68 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_kernel(const FwdParams p
     }
   }
   T* stage = reinterpret_cast<T*>(smem);
-  store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.o) + base(6), p.st[6][1], q0, p.Lq, tid,
-                              [&](int t, int i) { return O[t][i] * inv_l; });
+  // remainder columns: lane (i = lane % 16, w = lane / 16) holds head-dim 32*NMT + 4w .. +3 of query i (tile 0) / 16 + i (tile 1)
+  float inv16[2] = {inv_l, inv_l}, mun16[2] = {mu_n, mu_n};
+  if constexpr (TAIL) {
+    swap16f(inv_l, inv16[0], inv16[1]);
+    swap16f(mu_n, mun16[0], mun16[1]);
+  }
+  const int w16 = lane >> 4, i16 = lane & 15;
+  constexpr int OSTR = Cfg<T, D>::OSTRIDE, TAILW = D - 32 * NMT;
+  auto tail_o = [&](void* ws) {
+    if constexpr (TAIL) {
+      if (4 * w16 < TAILW) {
+#pragma unroll
+        for (int hq = 0; hq < 2; ++hq)
+          store4<T>(static_cast<T*>(ws) + (16 * hq + i16) * OSTR + 32 * NMT + 4 * w16, O16[hq][0] * inv16[hq], O16[hq][1] * inv16[hq],
+                    O16[hq][2] * inv16[hq], O16[hq][3] * inv16[hq]);
+      }
+    }
+  };
+  auto tail_to = [&](void* ws) {
+    if constexpr (TAIL && JVP) {
+      if (4 * w16 < TAILW) {
+#pragma unroll
+        for (int hq = 0; hq < 2; ++hq) {
+          float x[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[e] = fmaf(-mun16[hq], O16[hq][e] * inv16[hq], dO16[hq][e] * inv16[hq]);
+          store4<T>(static_cast<T*>(ws) + (16 * hq + i16) * OSTR + 32 * NMT + 4 * w16, x[0], x[1], x[2], x[3]);
+        }
+      }
+    }
+  };
+  store_rows_transposed<T, D, NW, NMT>(stage, reinterpret_cast<T*>(p.o) + base(6), p.st[6][1], q0, p.Lq, tid,
+                                       [&](int t, int i) { return O[t][i] * inv_l; }, tail_o);
   if constexpr (JVP)
-    store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.to) + base(7), p.st[7][1], q0, p.Lq, tid,
-                                [&](int t, int i) { return fmaf(-mu_n, O[t][i] * inv_l, dO[t][i] * inv_l); });
+    store_rows_transposed<T, D, NW, NMT>(stage, reinterpret_cast<T*>(p.to) + base(7), p.st[7][1], q0, p.Lq, tid,
+                                         [&](int t, int i) { return fmaf(-mu_n, O[t][i] * inv_l, dO[t][i] * inv_l); }, tail_to);
 }
 
-template <int D, bool JVP>
+template <int D, bool JVP, int NW>
 static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
   using F = FastCfg<D>;
   constexpr int tiles = 2 * (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES) + 512;
-  constexpr int stage = 128 * Cfg<__bf16, D>::OROWV * 16;
+  constexpr int stage = 32 * NW * Cfg<__bf16, D>::OROWV * 16;
   constexpr int smem = tiles > stage ? tiles : stage;
-  auto kern = attn_fwd_bf16_kernel<D, JVP>;
+  auto kern = attn_fwd_bf16_kernel<D, JVP, NW>;
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
       return -7;
     attr_set = true;
   }
-  const uint32_t nqb = (p.Lq + 127) / 128;
-  hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
+  const uint32_t nqb = (p.Lq + 32 * NW - 1) / (32 * NW);
+  hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(64 * NW), smem, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+// Work-group width policy (256-row work-groups when the sequence fills them).
+static bool fwd_wide_workgroups(int Lq) {
+  static const int force = [] { const char* e = getenv("DMF_ATTN_FWD_NW"); return e ? atoi(e) : 0; }();
+  if (force == 4) return false;
+  if (force == 8) return true;
+  return Lq > 128;
 }
 
 // Returns 1 if this translation unit has no kernel for the case (caller falls
@@ -313,13 +422,19 @@ int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_
   // 32-bit buffer addressing: every (batch, head) slab of K/V rows must span < 2 GiB
   const int64_t max_row = std::max(std::max(p.st[1][1], p.st[2][1]), jvp ? std::max(p.st[4][1], p.st[5][1]) : (int64_t)0);
   if (max_row * 2 * (int64_t)(p.Lkv + 32) >= (int64_t)1 << 31) return 1;
+  const bool wide = fwd_wide_workgroups(p.Lq);
+#define DMF_CASE(DD)                                                                           \
+  case DD:                                                                                     \
+    if (wide) return jvp ? launch_fast_t<DD, true, 8>(p, BH, stream) : launch_fast_t<DD, false, 8>(p, BH, stream); \
+    return jvp ? launch_fast_t<DD, true, 4>(p, BH, stream) : launch_fast_t<DD, false, 4>(p, BH, stream);
   switch (D) {
-    case 64: return jvp ? launch_fast_t<64, true>(p, BH, stream) : launch_fast_t<64, false>(p, BH, stream);
-    case 72: return jvp ? launch_fast_t<72, true>(p, BH, stream) : launch_fast_t<72, false>(p, BH, stream);
-    case 96: return jvp ? launch_fast_t<96, true>(p, BH, stream) : launch_fast_t<96, false>(p, BH, stream);
-    case 128: return jvp ? launch_fast_t<128, true>(p, BH, stream) : launch_fast_t<128, false>(p, BH, stream);
+    DMF_CASE(64)
+    DMF_CASE(72)
+    DMF_CASE(96)
+    DMF_CASE(128)
     default: return 1;
   }
+#undef DMF_CASE
 }
 
 }  // namespace dmf
