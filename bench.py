@@ -141,6 +141,22 @@ def cpu_baseline_config1():
     return out
 
 
+def mfma_probe():
+    """Sustained bf16 MFMA rate of this device from a register-only loop (dmf_amd/csrc/mfma_probe.hip):
+    with constant operands and with random operand bits (power-limited clocks)."""
+    import ctypes
+    path = os.path.join(ROOT, "dmf_amd", "libdmf_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.dmf_probe_mfma_tflops.restype = ctypes.c_float
+    lib.dmf_probe_mfma_tflops.argtypes = [ctypes.c_int, ctypes.c_int]
+    out = {}
+    for label, rnd in (("constant_operands_tflops", 0), ("random_operands_tflops", 1)):
+        out[label] = max(lib.dmf_probe_mfma_tflops(rnd, 100000) for _ in range(2))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -214,6 +230,7 @@ def main():
                              "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS}
             extra[wname] = row
             del ins
+        extra["mfma_probe"] = mfma_probe()
         try:
             from dmf_amd import harness
             extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10))

@@ -13,6 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdmf_attn.so")
+PROBE_LIB = os.path.join(HERE, "libdmf_probe.so")
 SOURCES = ["attn_fwd.hip", "attn_fwd_bf16.hip", "attn_bwd.hip", "attn_bwd_bf16.hip", "dmf_attn_abi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -46,6 +47,13 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
+    # measurement aid used by bench.py only (sustained MFMA rate probe); separate library, not part of the ABI
+    probe_obj = _compile("mfma_probe.hip", objdir)
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB, probe_obj], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr}")
+    if verbose:
+        print(f"built {PROBE_LIB}")
     return LIB
 
 

@@ -153,11 +153,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   const __amdgpu_buffer_rsrc_t rs_tv = make_rows_rsrc(JVP ? gtv : gv, JVP ? rb_tv : rb_v, p.Lkv, D * 2);
   auto issue = [&](int it) {
     const int s = it & 1;
-#ifdef DMF_EXP_SAMETILE
-    const uint32_t r0 = 0;
-#else
     const uint32_t r0 = (uint32_t)it * BKV;
-#endif
     issue_tile_rows<KP, VPR, NW>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
     issue_tile_rows<VP, VPR, NW>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
     if constexpr (JVP) {
@@ -170,12 +166,8 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   issue(0);
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile `it` has landed in LDS
-#ifndef DMF_EXP_NOBARRIER
     __syncthreads();                       // ... and everyone else's; also: all waves are done with the other stage
-#endif
-#ifndef DMF_EXP_NOLOAD
     if (it + 1 < ntiles) issue(it + 1);
-#endif
     const int s = it & 1;
 
     // ---- S^T (already scaled) and dS^T; the LDS reads of chunk c+1 are in
@@ -204,16 +196,13 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
         }
       });
     }
-    // ---- keys past the end (last tile only): their K/V rows were zero-filled, mask the scores
+    // ---- keys past the end: their K/V rows were zero-filled by the bounds check, mask the scores
     if ((it + 1) * BKV > p.Lkv) {
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         if (it * BKV + acc_row(i, g) >= p.Lkv) S[i] = -INFINITY;
     }
     // ---- lazy running maximum
-#ifdef DMF_EXP_NOSOFTMAX
-    f32x16 E = S, G = dS;
-#else
     float mx = fmaxf(S[0], S[1]);
 #pragma unroll
     for (int i = 2; i < 16; ++i) mx = fmaxf(mx, S[i]);
@@ -253,7 +242,6 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
         if constexpr (JVP) mu_run += G[i];
       }
     }
-#endif
     // ---- O^T += V^T P^T ; dO^T += V^T G^T + dV^T P^T, over 2*NMT operand groups
     //      (step st, head-dim tile t) plus, with TAIL, one 16-wide remainder group;
     //      group i+1 is read while group i multiplies
