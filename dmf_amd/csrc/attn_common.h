@@ -355,4 +355,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* bas
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (nrows - 1) * row_bytes + row_payload_bytes, 0x00020000);
 }
 
+// All NCHUNK 16-byte operand chunks of one row (this lane's row, half g) with
+// bounds-checked buffer loads issued back to back: rows past the end of the
+// resource read as zeros, chunk vectors past the head dim are zeroed here.
+template <int NCHUNK, int VPR>
+__device__ __forceinline__ void load_row_chunks(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_bytes, int row, int g, u32x4 (&out)[NCHUNK]) {
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c)
+    out[c] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (uint32_t)row * row_bytes + (2 * c + g) * 16, 0, 0));
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c)
+    if (2 * c + g >= VPR) out[c] = u32x4{0, 0, 0, 0};
+}
+
 }  // namespace dmf

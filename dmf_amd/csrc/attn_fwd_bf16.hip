@@ -76,6 +76,24 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   const T* gtk = JVP ? reinterpret_cast<const T*>(p.tk) + base(4) : nullptr;
   const T* gtv = JVP ? reinterpret_cast<const T*>(p.tv) + base(5) : nullptr;
 
+  const uint32_t rb_k = (uint32_t)p.st[1][1] * 2, rb_v = (uint32_t)p.st[2][1] * 2;
+  const uint32_t rb_tk = JVP ? (uint32_t)p.st[4][1] * 2 : 0, rb_tv = JVP ? (uint32_t)p.st[5][1] * 2 : 0;
+  const __amdgpu_buffer_rsrc_t rs_k = make_rows_rsrc(gk, rb_k, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_v = make_rows_rsrc(gv, rb_v, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_tk = make_rows_rsrc(JVP ? gtk : gk, JVP ? rb_tk : rb_k, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_tv = make_rows_rsrc(JVP ? gtv : gv, JVP ? rb_tv : rb_v, p.Lkv, D * 2);
+  auto issue = [&](int it) {
+    const int s = it & 1;
+    const uint32_t r0 = (uint32_t)it * BKV;
+    issue_tile_rows<KP, VPR, NW>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
+    issue_tile_rows<VP, VPR, NW>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
+    if constexpr (JVP) {
+      issue_tile_rows<KP, VPR, NW>(rs_tk, rb_tk, r0 * rb_tk, dKt(s), wave, lane);
+      issue_tile_rows<VP, VPR, NW>(rs_tv, rb_tv, r0 * rb_tv, dVt(s), wave, lane);
+    }
+  };
+
+
   // ---- padding of both stages: zeros, and the ones column of V
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
@@ -99,9 +117,12 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   u32x4 Qr[NCHUNK], dQr[JVP ? NCHUNK : 1];
   {
     const int qrow = q0 + wave * 32 + c32;
-    const bool ok = qrow < p.Lq;
-    const T* gq = reinterpret_cast<const T*>(p.q) + base(0) + (int64_t)qrow * p.st[0][1];
-    const T* gtq = JVP ? reinterpret_cast<const T*>(p.tq) + base(3) + (int64_t)qrow * p.st[3][1] : nullptr;
+    const uint32_t rb_q = (uint32_t)p.st[0][1] * 2;
+    load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(0), rb_q, p.Lq, D * 2), rb_q, qrow, g, Qr);
+    if constexpr (JVP) {
+      const uint32_t rb_tq = (uint32_t)p.st[3][1] * 2;
+      load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.tq) + base(3), rb_tq, p.Lq, D * 2), rb_tq, qrow, g, dQr);
+    }
     auto scaled = [&](u32x4 x) {
       u32x4 y;
 #pragma unroll
@@ -111,12 +132,13 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
     };
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
-      const int cv = 2 * c + g;
-      const bool in = ok && cv < VPR;
-      Qr[c] = in ? scaled(*reinterpret_cast<const u32x4*>(gq + cv * 8)) : u32x4{0, 0, 0, 0};
-      if constexpr (JVP) dQr[c] = in ? scaled(*reinterpret_cast<const u32x4*>(gtq + cv * 8)) : u32x4{0, 0, 0, 0};
+      Qr[c] = scaled(Qr[c]);
+      if constexpr (JVP) dQr[c] = scaled(dQr[c]);
     }
   }
+
+  // first key tile on its way (issued after the Q loads: measured faster than issuing it first)
+  issue(0);
 
   constexpr int NMT = F::NMT;
   constexpr bool TAIL = F::TAIL;
@@ -145,25 +167,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   const uint32_t t_lane_addr = lds_addr(smem) + F::KBYTES +
       ((16 * ((lane >> 4) & 1) + 4 * (lane >> 5) + ((lane & 15) >> 2)) * VSTR + 32 * F::NMT + 4 * (lane & 3)) * 2;
 
-  const uint32_t rb_k = (uint32_t)p.st[1][1] * 2, rb_v = (uint32_t)p.st[2][1] * 2;
-  const uint32_t rb_tk = JVP ? (uint32_t)p.st[4][1] * 2 : 0, rb_tv = JVP ? (uint32_t)p.st[5][1] * 2 : 0;
-  const __amdgpu_buffer_rsrc_t rs_k = make_rows_rsrc(gk, rb_k, p.Lkv, D * 2);
-  const __amdgpu_buffer_rsrc_t rs_v = make_rows_rsrc(gv, rb_v, p.Lkv, D * 2);
-  const __amdgpu_buffer_rsrc_t rs_tk = make_rows_rsrc(JVP ? gtk : gk, JVP ? rb_tk : rb_k, p.Lkv, D * 2);
-  const __amdgpu_buffer_rsrc_t rs_tv = make_rows_rsrc(JVP ? gtv : gv, JVP ? rb_tv : rb_v, p.Lkv, D * 2);
-  auto issue = [&](int it) {
-    const int s = it & 1;
-    const uint32_t r0 = (uint32_t)it * BKV;
-    issue_tile_rows<KP, VPR, NW>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
-    issue_tile_rows<VP, VPR, NW>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
-    if constexpr (JVP) {
-      issue_tile_rows<KP, VPR, NW>(rs_tk, rb_tk, r0 * rb_tk, dKt(s), wave, lane);
-      issue_tile_rows<VP, VPR, NW>(rs_tv, rb_tv, r0 * rb_tv, dVt(s), wave, lane);
-    }
-  };
-
   const int ntiles = (p.Lkv + BKV - 1) / BKV;
-  issue(0);
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile `it` has landed in LDS
     __syncthreads();                       // ... and everyone else's; also: all waves are done with the other stage
@@ -408,8 +412,9 @@ static bool fwd_wide_workgroups(int Lq) {
 // back to the generic kernel), else 0 / negative error code.
 int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_t stream) {
   // 32-bit buffer addressing: every (batch, head) slab of K/V rows must span < 2 GiB
-  const int64_t max_row = std::max(std::max(p.st[1][1], p.st[2][1]), jvp ? std::max(p.st[4][1], p.st[5][1]) : (int64_t)0);
-  if (max_row * 2 * (int64_t)(p.Lkv + 32) >= (int64_t)1 << 31) return 1;
+  int64_t max_row = std::max(std::max(p.st[0][1], p.st[1][1]), p.st[2][1]);
+  if (jvp) max_row = std::max(max_row, std::max(std::max(p.st[3][1], p.st[4][1]), p.st[5][1]));
+  if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 256) >= (int64_t)1 << 31) return 1;
   const bool wide = fwd_wide_workgroups(p.Lq);
 #define DMF_CASE(DD)                                                                           \
   case DD:                                                                                     \
