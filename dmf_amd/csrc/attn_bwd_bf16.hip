@@ -20,6 +20,8 @@ struct BwdFastCfg {
   static constexpr int STR = P * 8;
   static constexpr int TBYTES = 32 * P * 16;          // one 32-row tile
   static constexpr int STAT = 256;                    // per stage: 32 x lse, 32 x delta (fp32)
+  static constexpr bool TAIL = (D % 32) != 0 && (D % 32) <= 16;   // 16-wide remainder via 16x16x32 MFMAs (72, 80)
+  static constexpr int NMT = TAIL ? D / 32 : NDT;                 // full 32-wide output tiles
 };
 
 // bf16x8 chunk times a scalar, re-rounded to bf16.
@@ -46,7 +48,8 @@ template <int D>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParams p) {
   using F = BwdFastCfg<D>;
   using T = __bf16;
-  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NDT = F::NDT, P = F::P, STR = F::STR;
+  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR;
+  constexpr bool TAIL = F::TAIL;
   constexpr int STAGE = 2 * F::TBYTES;   // K | V
   constexpr int V_OFF = F::TBYTES;
 
@@ -70,20 +73,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
   u32x4 Qr[NCHUNK], dOr[NCHUNK];
   float dpart = 0.f;
   {
-    const T* gq = reinterpret_cast<const T*>(p.q) + base(1) + (int64_t)qrow * p.st[1][1];
-    const T* gdo = reinterpret_cast<const T*>(p.dout) + base(0) + (int64_t)qrow * p.st[0][1];
-    const T* go = reinterpret_cast<const T*>(p.o) + base(4) + (int64_t)qrow * p.st[4][1];
+    u32x4 Or[NCHUNK];
+    const uint32_t rb_q = (uint32_t)p.st[1][1] * 2, rb_do = (uint32_t)p.st[0][1] * 2, rb_o = (uint32_t)p.st[4][1] * 2;
+    load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(1), rb_q, p.Lq, D * 2), rb_q, qrow, g, Qr);
+    load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.dout) + base(0), rb_do, p.Lq, D * 2), rb_do, qrow, g, dOr);
+    load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.o) + base(4), rb_o, p.Lq, D * 2), rb_o, qrow, g, Or);
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
-      const int cv = 2 * c + g;
-      const bool in = qok && cv < VPR;
-      Qr[c] = in ? scale_bf16x8(*reinterpret_cast<const u32x4*>(gq + cv * 8), p.scale_log2) : u32x4{0, 0, 0, 0};
-      dOr[c] = in ? *reinterpret_cast<const u32x4*>(gdo + cv * 8) : u32x4{0, 0, 0, 0};
-      const u32x4 ov = in ? *reinterpret_cast<const u32x4*>(go + cv * 8) : u32x4{0, 0, 0, 0};
+      Qr[c] = scale_bf16x8(Qr[c], p.scale_log2);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        dpart += __uint_as_float(dOr[c][e] << 16) * __uint_as_float(ov[e] << 16);
-        dpart += __uint_as_float(dOr[c][e] & 0xffff0000u) * __uint_as_float(ov[e] & 0xffff0000u);
+        dpart += __uint_as_float(dOr[c][e] << 16) * __uint_as_float(Or[c][e] << 16);
+        dpart += __uint_as_float(dOr[c][e] & 0xffff0000u) * __uint_as_float(Or[c][e] & 0xffff0000u);
       }
     }
   }
@@ -94,9 +95,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
     if (g == 0) p.delta[(int64_t)bh * p.Lq + qrow] = delta;
   }
 
-  f32x16 dQ[NDT];
+  f32x16 dQ[NMT];
+  f32x4 dQ16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
 #pragma unroll
-  for (int t = 0; t < NDT; ++t) dQ[t] = f32x16{0};
+  for (int t = 0; t < NMT; ++t) dQ[t] = f32x16{0};
 
   const uint32_t rb_k = (uint32_t)p.st[2][1] * 2, rb_v = (uint32_t)p.st[3][1] * 2;
   const __amdgpu_buffer_rsrc_t rs_k = make_rows_rsrc(reinterpret_cast<const T*>(p.k) + base(2), rb_k, p.Lkv, D * 2);
@@ -108,6 +110,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
   };
   const uint32_t row_addr = lds_addr(smem) + c32 * STR * 2 + g * 16;
   const uint32_t col_addr = lds_addr(smem) + ((4 * g + ((lane & 15) >> 2)) * STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  const uint32_t tail_addr = lds_addr(smem) + tail_lane_offset(lane, STR, 32 * NMT) * 2;
 
   const int ntiles = (p.Lkv + 31) / 32;
   issue(0);
@@ -147,21 +151,32 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
     // ---- dQ^T += K^T dS^T
     {
       ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
-      constexpr int NG = 2 * NDT;
+      constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
       TrPair kk[2];
-      auto lo_off = [](int gi) constexpr { return (16 * (gi / NDT) * STR + 32 * (gi % NDT)) * 2; };
+      auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
       kk[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
-      static_for<NG>([&](auto gc) {
+      static_for<NGT>([&](auto gc) {
         constexpr int gi = decltype(gc)::value;
-        constexpr bool more = gi + 1 < NG;
-        if constexpr (more) kk[(gi + 1) & 1] = lds_tr16_issue<lo_off(gi + 1), lo_off(gi + 1) + 8 * STR * 2>(ca);
+        constexpr bool more = gi + 1 < NGT;
+        if constexpr (gi + 1 < NG) kk[(gi + 1) & 1] = lds_tr16_issue<lo_off(gi + 1), lo_off(gi + 1) + 8 * STR * 2>(ca);
+        else if constexpr (more) kk[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(tail_addr + (it & 1) * STAGE);
         lds_tr16_wait<more ? 2 : 0>(kk[gi & 1]);
-        mma_col<T>(dQ[gi % NDT], tr_operand(kk[gi & 1]), ds[gi / NDT]);
+        if constexpr (gi < NG) {
+          mma_col<T>(dQ[gi % NMT], tr_operand(kk[gi & 1]), ds[gi / NMT]);
+        } else {
+          ColOperand d0, d1;
+          tail_operands(ds[0], ds[1], d0, d1);
+          mma16(dQ16[0], tr_operand(kk[gi & 1]), d0);
+          mma16(dQ16[1], tr_operand(kk[gi & 1]), d1);
+        }
       });
     }
   }
-  store_rows_transposed<T, D>(reinterpret_cast<T*>(smem), reinterpret_cast<T*>(p.dq) + base(5), p.st[5][1], q0, p.Lq, tid,
-                              [&](int t, int i) { return dQ[t][i] * p.scale; });
+  store_rows_transposed<T, D, 4, NMT>(reinterpret_cast<T*>(smem), reinterpret_cast<T*>(p.dq) + base(5), p.st[5][1], q0, p.Lq, tid,
+                                      [&](int t, int i) { return dQ[t][i] * p.scale; },
+                                      [&](void* ws) {
+                                        if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dQ16[hq][e] * p.scale; });
+                                      });
 }
 
 // --------------------------------------------------------------- dK/dV kernel
@@ -169,7 +184,8 @@ template <int D>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdParams p) {
   using F = BwdFastCfg<D>;
   using T = __bf16;
-  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NDT = F::NDT, P = F::P, STR = F::STR;
+  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR;
+  constexpr bool TAIL = F::TAIL;
   constexpr int STAGE = 2 * F::TBYTES + F::STAT;   // Q | dout | lse[32], delta[32]
   constexpr int DO_OFF = F::TBYTES, STAT_OFF = 2 * F::TBYTES;
 
@@ -191,20 +207,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   u32x4 Kr[NCHUNK], Vr[NCHUNK];
   {
     const int krow = k0 + wave * 32 + c32;
-    const bool ok = krow < p.Lkv;
-    const T* gk = reinterpret_cast<const T*>(p.k) + base(2) + (int64_t)krow * p.st[2][1];
-    const T* gv = reinterpret_cast<const T*>(p.v) + base(3) + (int64_t)krow * p.st[3][1];
+    const uint32_t rb_k = (uint32_t)p.st[2][1] * 2, rb_v = (uint32_t)p.st[3][1] * 2;
+    load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.k) + base(2), rb_k, p.Lkv, D * 2), rb_k, krow, g, Kr);
+    load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.v) + base(3), rb_v, p.Lkv, D * 2), rb_v, krow, g, Vr);
 #pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) {
-      const int cv = 2 * c + g;
-      const bool in = ok && cv < VPR;
-      Kr[c] = in ? scale_bf16x8(*reinterpret_cast<const u32x4*>(gk + cv * 8), p.scale_log2) : u32x4{0, 0, 0, 0};
-      Vr[c] = in ? *reinterpret_cast<const u32x4*>(gv + cv * 8) : u32x4{0, 0, 0, 0};
-    }
+    for (int c = 0; c < NCHUNK; ++c) Kr[c] = scale_bf16x8(Kr[c], p.scale_log2);
   }
-  f32x16 dK[NDT], dV[NDT];
+  f32x16 dK[NMT], dV[NMT];
+  f32x4 dK16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}}, dV16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
 #pragma unroll
-  for (int t = 0; t < NDT; ++t) {
+  for (int t = 0; t < NMT; ++t) {
     dK[t] = f32x16{0};
     dV[t] = f32x16{0};
   }
@@ -226,6 +238,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   };
   const uint32_t row_addr = lds_addr(smem) + c32 * STR * 2 + g * 16;
   const uint32_t col_addr = lds_addr(smem) + ((4 * g + ((lane & 15) >> 2)) * STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  const uint32_t tail_addr = lds_addr(smem) + tail_lane_offset(lane, STR, 32 * NMT) * 2;
 
   const int ntiles = (p.Lq + 31) / 32;
   issue(0);
@@ -271,30 +285,50 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     {
       ColOperand pp[2] = {acc_operand<T>(Pm, 0), acc_operand<T>(Pm, 1)};
       ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
-      constexpr int NG = 2 * NDT;
+      constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
       TrPair qq[2], oo[2];
-      auto lo_off = [](int gi) constexpr { return (16 * (gi / NDT) * STR + 32 * (gi % NDT)) * 2; };
+      auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
       qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
       oo[0] = lds_tr16_issue<lo_off(0) + DO_OFF, lo_off(0) + 8 * STR * 2 + DO_OFF>(ca);
-      static_for<NG>([&](auto gc) {
+      static_for<NGT>([&](auto gc) {
         constexpr int gi = decltype(gc)::value;
-        constexpr bool more = gi + 1 < NG;
-        if constexpr (more) {
+        constexpr bool more = gi + 1 < NGT;
+        if constexpr (gi + 1 < NG) {
           constexpr int LO = lo_off(gi + 1), HI = LO + 8 * STR * 2;
           qq[(gi + 1) & 1] = lds_tr16_issue<LO, HI>(ca);
           oo[(gi + 1) & 1] = lds_tr16_issue<LO + DO_OFF, HI + DO_OFF>(ca);
+        } else if constexpr (more) {
+          const uint32_t ta = tail_addr + (it & 1) * STAGE;
+          qq[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(ta);
+          oo[(gi + 1) & 1] = lds_tr16_issue<DO_OFF, 8 * STR * 2 + DO_OFF>(ta);
         }
         lds_tr16_wait<more ? 4 : 0>(qq[gi & 1], oo[gi & 1]);
-        mma_col<T>(dV[gi % NDT], tr_operand(oo[gi & 1]), pp[gi / NDT]);
-        mma_col<T>(dK[gi % NDT], tr_operand(qq[gi & 1]), ds[gi / NDT]);
+        if constexpr (gi < NG) {
+          mma_col<T>(dV[gi % NMT], tr_operand(oo[gi & 1]), pp[gi / NMT]);
+          mma_col<T>(dK[gi % NMT], tr_operand(qq[gi & 1]), ds[gi / NMT]);
+        } else {
+          ColOperand p0, p1, d0, d1;
+          tail_operands(pp[0], pp[1], p0, p1);
+          tail_operands(ds[0], ds[1], d0, d1);
+          mma16(dV16[0], tr_operand(oo[gi & 1]), p0);
+          mma16(dV16[1], tr_operand(oo[gi & 1]), p1);
+          mma16(dK16[0], tr_operand(qq[gi & 1]), d0);
+          mma16(dK16[1], tr_operand(qq[gi & 1]), d1);
+        }
       });
     }
   }
   T* stage = reinterpret_cast<T*>(smem);
-  store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.dk) + base(6), p.st[6][1], k0, p.Lkv, tid,
-                              [&](int t, int i) { return dK[t][i] * p.scale; });
-  store_rows_transposed<T, D>(stage, reinterpret_cast<T*>(p.dv) + base(7), p.st[7][1], k0, p.Lkv, tid,
-                              [&](int t, int i) { return dV[t][i]; });
+  store_rows_transposed<T, D, 4, NMT>(stage, reinterpret_cast<T*>(p.dk) + base(6), p.st[6][1], k0, p.Lkv, tid,
+                                      [&](int t, int i) { return dK[t][i] * p.scale; },
+                                      [&](void* ws) {
+                                        if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dK16[hq][e] * p.scale; });
+                                      });
+  store_rows_transposed<T, D, 4, NMT>(stage, reinterpret_cast<T*>(p.dv) + base(7), p.st[7][1], k0, p.Lkv, tid,
+                                      [&](int t, int i) { return dV[t][i]; },
+                                      [&](void* ws) {
+                                        if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dV16[hq][e]; });
+                                      });
 }
 
 template <int D>
@@ -322,8 +356,8 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
 // Returns 1 if there is no tuned kernel for the case (caller uses the generic ones).
 int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream) {
   // 32-bit buffer addressing: every (batch, head) slab of rows must span < 2 GiB
-  const int64_t max_row = std::max(std::max(p.st[0][1], p.st[1][1]), std::max(p.st[2][1], p.st[3][1]));
-  if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 32) >= (int64_t)1 << 31) return 1;
+  const int64_t max_row = std::max(std::max(std::max(p.st[0][1], p.st[1][1]), std::max(p.st[2][1], p.st[3][1])), p.st[4][1]);
+  if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 256) >= (int64_t)1 << 31) return 1;
   switch (D) {
     case 64: return launch_bwd_fast_t<64>(p, BH, stream);
     case 72: return launch_bwd_fast_t<72>(p, BH, stream);

@@ -355,6 +355,40 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* bas
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (nrows - 1) * row_bytes + row_payload_bytes, 0x00020000);
 }
 
+// Epilogue of the 16-wide remainder tiles (head dims 72, 80): lane (i = lane % 16,
+// w = lane / 16) holds head-dim columns 32*NMT + 4w .. +3 of row i (tile 0) and of
+// row 16 + i (tile 1) of this wave's 32 rows; value(hq, e) supplies the numbers.
+// `ws` = staging row 0 of this wave (see store_rows_transposed).
+template <typename T, int D, int NMT, typename VF>
+__device__ __forceinline__ void store_tail16(void* ws, int lane, VF value) {
+  constexpr int OSTR = Cfg<T, D>::OSTRIDE, TAILW = D - 32 * NMT;
+  const int w16 = lane >> 4, i16 = lane & 15;
+  if (4 * w16 < TAILW) {
+#pragma unroll
+    for (int hq = 0; hq < 2; ++hq)
+      store4<T>(static_cast<T*>(ws) + (16 * hq + i16) * OSTR + 32 * NMT + 4 * w16, value(hq, 0), value(hq, 1), value(hq, 2), value(hq, 3));
+  }
+}
+
+// Both B operands (query/key halves 0 and 1) of the 16x16x32 remainder products
+// from the two 32x32x16-layout operands of a 32-row tile (steps 0 and 1).
+__device__ __forceinline__ void tail_operands(const ColOperand& st0, const ColOperand& st1, ColOperand& half0, ColOperand& half1) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    uint32_t ev, od;
+    swap16(st0.v[r], st1.v[r], ev, od);
+    half0.v[r] = ev;
+    half1.v[r] = od;
+  }
+}
+
+// Lane offset (in elements) for the transposed remainder operand inside a
+// row-major 32-row tile of pitch STR: 16-lane row w covers tile rows
+// 16*(w%2) + 4*(w/2) + {0..3, 8..11} at columns col0 .. col0+15.
+__device__ __forceinline__ int tail_lane_offset(int lane, int STR, int col0) {
+  return (16 * ((lane >> 4) & 1) + 4 * (lane >> 5) + ((lane & 15) >> 2)) * STR + col0 + 4 * (lane & 3);
+}
+
 // All NCHUNK 16-byte operand chunks of one row (this lane's row, half g) with
 // bounds-checked buffer loads issued back to back: rows past the end of the
 // resource read as zeros, chunk vectors past the head dim are zeroed here.

@@ -164,8 +164,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
       lds_addr(smem) + F::KBYTES + ((4 * g + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
   // Remainder (16x16x32) operand: 16-lane row w covers keys 16*(w%2) + 4*(w/2) + {0..3, 8..11} -- the keys whose
   // probabilities that row receives from swap16 -- at head-dim columns 32*NMT .. 32*NMT+15.
-  const uint32_t t_lane_addr = lds_addr(smem) + F::KBYTES +
-      ((16 * ((lane >> 4) & 1) + 4 * (lane >> 5) + ((lane & 15) >> 2)) * VSTR + 32 * F::NMT + 4 * (lane & 3)) * 2;
+  const uint32_t t_lane_addr = lds_addr(smem) + F::KBYTES + tail_lane_offset(lane, VSTR, 32 * F::NMT) * 2;
 
   const int ntiles = (p.Lkv + BKV - 1) / BKV;
   for (int it = 0; it < ntiles; ++it) {
@@ -286,18 +285,8 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
         } else {
           // B operands for the two query halves: lanes of 16-lane row w take (half g = w/2, step st = w%2)
           ColOperand pe0, pe1, pg0, pg1;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            uint32_t ev, od;
-            swap16(pe[0].v[r], pe[1].v[r], ev, od);
-            pe0.v[r] = ev;
-            pe1.v[r] = od;
-            if constexpr (JVP) {
-              swap16(pg[0].v[r], pg[1].v[r], ev, od);
-              pg0.v[r] = ev;
-              pg1.v[r] = od;
-            }
-          }
+          tail_operands(pe[0], pe[1], pe0, pe1);
+          if constexpr (JVP) tail_operands(pg[0], pg[1], pg0, pg1);
           mma16(O16[0], tr_operand(v[gi & 1]), pe0);
           mma16(O16[1], tr_operand(v[gi & 1]), pe1);
           if constexpr (JVP) {
@@ -350,30 +339,12 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
     swap16f(inv_l, inv16[0], inv16[1]);
     swap16f(mu_n, mun16[0], mun16[1]);
   }
-  const int w16 = lane >> 4, i16 = lane & 15;
-  constexpr int OSTR = Cfg<T, D>::OSTRIDE, TAILW = D - 32 * NMT;
   auto tail_o = [&](void* ws) {
-    if constexpr (TAIL) {
-      if (4 * w16 < TAILW) {
-#pragma unroll
-        for (int hq = 0; hq < 2; ++hq)
-          store4<T>(static_cast<T*>(ws) + (16 * hq + i16) * OSTR + 32 * NMT + 4 * w16, O16[hq][0] * inv16[hq], O16[hq][1] * inv16[hq],
-                    O16[hq][2] * inv16[hq], O16[hq][3] * inv16[hq]);
-      }
-    }
+    if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return O16[hq][e] * inv16[hq]; });
   };
   auto tail_to = [&](void* ws) {
-    if constexpr (TAIL && JVP) {
-      if (4 * w16 < TAILW) {
-#pragma unroll
-        for (int hq = 0; hq < 2; ++hq) {
-          float x[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) x[e] = fmaf(-mun16[hq], O16[hq][e] * inv16[hq], dO16[hq][e] * inv16[hq]);
-          store4<T>(static_cast<T*>(ws) + (16 * hq + i16) * OSTR + 32 * NMT + 4 * w16, x[0], x[1], x[2], x[3]);
-        }
-      }
-    }
+    if constexpr (TAIL && JVP)
+      store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return fmaf(-mun16[hq], O16[hq][e] * inv16[hq], dO16[hq][e] * inv16[hq]); });
   };
   store_rows_transposed<T, D, NW, NMT>(stage, reinterpret_cast<T*>(p.o) + base(6), p.st[6][1], q0, p.Lq, tid,
                                        [&](int t, int i) { return O[t][i] * inv_l; }, tail_o);
