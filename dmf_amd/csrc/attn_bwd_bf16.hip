@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
   issue(0);
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-    __syncthreads();
+    lds_barrier();
     if (it + 1 < ntiles) issue(it + 1);
     const uint32_t ra = row_addr + (it & 1) * STAGE, ca = col_addr + (it & 1) * STAGE;
 
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   issue(0);
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-    __syncthreads();
+    lds_barrier();
     if (it + 1 < ntiles) issue(it + 1);
     const uint32_t ra = row_addr + (it & 1) * STAGE, ca = col_addr + (it & 1) * STAGE;
     const float* stat = reinterpret_cast<const float*>(smem + (it & 1) * STAGE + STAT_OFF);

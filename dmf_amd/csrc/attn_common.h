@@ -234,6 +234,15 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t id, uint32_t total) {
   return (id % kXcd) * (total / kXcd) + id / kXcd;
 }
 
+// Work-group barrier that orders LDS traffic only.  __syncthreads() also makes
+// prior *global* stores visible, i.e. waits until they are acknowledged -- which
+// stalls an epilogue for microseconds when output rows have just been stored.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // Convert four consecutive fp32 values to T and store them to LDS.
 template <typename T>
 __device__ __forceinline__ void store4(T* dst, float a, float b, float c, float d) {
@@ -305,12 +314,11 @@ __device__ __forceinline__ void zero_tile_padding(T* tile, int tid) {
 // staging row 0 of this wave, row pitch Cfg::OSTRIDE).
 struct NoTail { __device__ __forceinline__ void operator()(void*) const {} };
 
-template <typename T, int D, int NW = 4, int NMAIN = Cfg<T, D>::NDT, typename F, typename TF = NoTail>
-__device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t row_stride, int row0, int nrows, int tid, F value,
-                                                      TF tail = TF{}) {
+// Part 1: write the scaled accumulators into the staging rows of this wave (no barrier, no global traffic).
+template <typename T, int D, int NMAIN = Cfg<T, D>::NDT, typename F, typename TF = NoTail>
+__device__ __forceinline__ void stage_rows(T* stage, int tid, F value, TF tail = TF{}) {
   using C = Cfg<T, D>;
   const int lane = tid & 63, wave = tid >> 6, c32 = lane & 31, g = lane >> 5;
-  __syncthreads();
   T* srow = stage + (wave * 32 + c32) * C::OSTRIDE;
 #pragma unroll
   for (int t = 0; t < NMAIN; ++t)
@@ -318,13 +326,29 @@ __device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t
     for (int j = 0; j < 4; ++j)
       store4<T>(srow + t * 32 + j * 8 + 4 * g, value(t, 4 * j), value(t, 4 * j + 1), value(t, 4 * j + 2), value(t, 4 * j + 3));
   tail(stage + wave * 32 * C::OSTRIDE);
-  __syncthreads();
-  for (int v = tid; v < 32 * NW * C::VPR; v += 64 * NW) {
-    const int row = v / C::VPR, cv = v % C::VPR;
-    if (row0 + row < nrows)
-      *reinterpret_cast<u32x4*>(gdst + (int64_t)(row0 + row) * row_stride + cv * C::VEC) =
-          *reinterpret_cast<const u32x4*>(stage + row * C::OSTRIDE + cv * C::VEC);
-  }
+}
+// Part 2: "round" r of the coalesced copy staging -> global: every thread moves one 16-byte vector.
+// Rounds 0 .. store_rounds()-1 cover the 32*NW staged rows.
+template <typename T, int D, int NW>
+__device__ __forceinline__ constexpr int store_rounds() { return (32 * NW * Cfg<T, D>::VPR + 64 * NW - 1) / (64 * NW); }
+
+template <typename T, int D, int NW>
+__device__ __forceinline__ void store_staged_round(const T* stage, T* gdst, int64_t row_stride, int row0, int nrows, int tid, int r) {
+  using C = Cfg<T, D>;
+  const int v = tid + r * 64 * NW;
+  const int row = v / C::VPR, cv = v % C::VPR;
+  if (v < 32 * NW * C::VPR && row0 + row < nrows)
+    *reinterpret_cast<u32x4*>(gdst + (int64_t)(row0 + row) * row_stride + cv * C::VEC) =
+        *reinterpret_cast<const u32x4*>(stage + row * C::OSTRIDE + cv * C::VEC);
+}
+
+template <typename T, int D, int NW = 4, int NMAIN = Cfg<T, D>::NDT, typename F, typename TF = NoTail>
+__device__ __forceinline__ void store_rows_transposed(T* stage, T* gdst, int64_t row_stride, int row0, int nrows, int tid, F value,
+                                                      TF tail = TF{}) {
+  lds_barrier();
+  stage_rows<T, D, NMAIN>(stage, tid, value, tail);
+  lds_barrier();
+  for (int r = 0; r < store_rounds<T, D, NW>(); ++r) store_staged_round<T, D, NW>(stage, gdst, row_stride, row0, nrows, tid, r);
 }
 
 // Issue the HBM -> LDS loads of one tensor tile (32 rows): wave w of the NW waves
@@ -394,12 +418,13 @@ __device__ __forceinline__ int tail_lane_offset(int lane, int STR, int col0) {
 // resource read as zeros, chunk vectors past the head dim are zeroed here.
 template <int NCHUNK, int VPR>
 __device__ __forceinline__ void load_row_chunks(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_bytes, int row, int g, u32x4 (&out)[NCHUNK]) {
+  // A chunk vector past the head dim gets an out-of-range offset, so the bounds check zero-fills it too and the
+  // loaded registers need no fix-up (a fix-up would make the caller wait for the data right here).
 #pragma unroll
-  for (int c = 0; c < NCHUNK; ++c)
-    out[c] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (uint32_t)row * row_bytes + (2 * c + g) * 16, 0, 0));
-#pragma unroll
-  for (int c = 0; c < NCHUNK; ++c)
-    if (2 * c + g >= VPR) out[c] = u32x4{0, 0, 0, 0};
+  for (int c = 0; c < NCHUNK; ++c) {
+    const uint32_t off = (2 * c + g < VPR) ? (uint32_t)row * row_bytes + (2 * c + g) * 16 : 0x7ffffff0u;
+    out[c] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
+  }
 }
 
 }  // namespace dmf

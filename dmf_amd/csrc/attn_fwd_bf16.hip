@@ -169,7 +169,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   const int ntiles = (p.Lkv + BKV - 1) / BKV;
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile `it` has landed in LDS
-    __syncthreads();                       // ... and everyone else's; also: all waves are done with the other stage
+    lds_barrier();                         // ... and everyone else's; also: all waves are done with the other stage
     if (it + 1 < ntiles) issue(it + 1);
     const int s = it & 1;
 
