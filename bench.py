@@ -141,9 +141,10 @@ def cpu_baseline_config1():
     return out
 
 
-def mfma_probe():
-    """Sustained bf16 MFMA rate of this device from a register-only loop (dmf_amd/csrc/mfma_probe.hip):
-    with constant operands and with random operand bits (power-limited clocks)."""
+def device_probes():
+    """Practical ceilings of this device (dmf_amd/csrc/probes.hip): sustained bf16 MFMA rate from a register-only
+    loop with constant and with random operand bits (power-limited clocks), and the bandwidth of a math-free kernel
+    with the operator's row access pattern at the N=256 workload."""
     import ctypes
     path = os.path.join(ROOT, "dmf_amd", "libdmf_probe.so")
     if not os.path.exists(path):
@@ -152,8 +153,14 @@ def mfma_probe():
     lib.dmf_probe_mfma_tflops.restype = ctypes.c_float
     lib.dmf_probe_mfma_tflops.argtypes = [ctypes.c_int, ctypes.c_int]
     out = {}
-    for label, rnd in (("constant_operands_tflops", 0), ("random_operands_tflops", 1)):
+    for label, rnd in (("mfma_constant_operands_tflops", 0), ("mfma_random_operands_tflops", 1)):
         out[label] = max(lib.dmf_probe_mfma_tflops(rnd, 100000) for _ in range(2))
+    # memory-system ceiling for the operator's access pattern (6 reads + 2 writes of D-wide rows per head, no math)
+    lib.dmf_probe_rows_stream_tbps.restype = ctypes.c_float
+    lib.dmf_probe_rows_stream_tbps.argtypes = [ctypes.c_int] * 5
+    B, H, N, D, _ = WORKLOADS["xl2_256px"]
+    out["rows_stream_BNHD_tbps"] = lib.dmf_probe_rows_stream_tbps(B, H, N, D, 0)
+    out["rows_stream_head_contiguous_tbps"] = lib.dmf_probe_rows_stream_tbps(B, H, N, D, 1)
     return out
 
 
@@ -205,7 +212,7 @@ def main():
                    "wall_ms_per_step": wall_ms},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name),
-                     "kernel": "dmf::attn_fwd_bf16_kernel<72, true>",
+                     "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8>",
                      "hbm_gbs_algorithmic": attn_bytes(B, H, N, D, "fwd_jvp") / (ms * 1e-3) / 1e9},
     }
 
@@ -230,7 +237,7 @@ def main():
                              "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS}
             extra[wname] = row
             del ins
-        extra["mfma_probe"] = mfma_probe()
+        extra["device_probes"] = device_probes()
         try:
             from dmf_amd import harness
             extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10))

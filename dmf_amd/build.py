@@ -47,8 +47,8 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
-    # measurement aid used by bench.py only (sustained MFMA rate probe); separate library, not part of the ABI
-    probe_obj = _compile("mfma_probe.hip", objdir)
+    # measurement aids used by bench.py only (sustained MFMA rate, row-streaming bandwidth); separate library, not part of the ABI
+    probe_obj = _compile("probes.hip", objdir)
     r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB, probe_obj], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
