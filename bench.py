@@ -31,8 +31,8 @@ if ROOT not in sys.path:
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the fused fwd+JVP kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (each scaled by what the counter reads for a plain 1 GiB copy; summary in profiles/attn_fwd_jvp_bf16_d72_xl2_512px.txt)
-MEASURED_TRAFFIC_BYTES = {"xl2_512px": 1.2768e9}
+# (each scaled by what the counter reads for a plain 1 GiB copy; summaries in profiles/attn_fwd_jvp_bf16_d72_*.txt)
+MEASURED_TRAFFIC_BYTES = {"xl2_512px": 1.2129e9, "xl2_256px": 1.2125e9}
 
 WORKLOADS = {
     # name: (B, H, N, D, qk_norm)
