@@ -339,13 +339,8 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
   constexpr int smem = tiles > stage ? tiles : stage;
   auto k1 = attn_bwd_dq_bf16_kernel<D>;
   auto k2 = attn_bwd_dkv_bf16_kernel<D>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
-      return -7;
-    attr_set = true;
-  }
+  static bool lds_ok1[64] = {}, lds_ok2[64] = {};
+  if (!ensure_dynamic_lds(k1, smem, lds_ok1) || !ensure_dynamic_lds(k2, smem, lds_ok2)) return -7;
   const uint32_t nqb = (p.Lq + 127) / 128, nkb = (p.Lkv + 127) / 128;
   hipLaunchKernelGGL(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
   if (hipGetLastError() != hipSuccess) return -7;

@@ -199,12 +199,8 @@ static int launch_fwd_t(const FwdParams& p, int BH, hipStream_t stream) {
   constexpr int stage = 128 * C::OROWV * 16;
   constexpr int smem = tiles > stage ? tiles : stage;
   auto kern = attn_fwd_kernel<T, D, JVP>;
-  static bool attr_set = false;   // idempotent; a benign race at worst repeats the call
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
-      return -7;
-    attr_set = true;
-  }
+  static bool lds_ok[64] = {};
+  if (!ensure_dynamic_lds(kern, smem, lds_ok)) return -7;
   const uint32_t nqb = (p.Lq + 127) / 128;
   hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : -7;

@@ -360,12 +360,8 @@ static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
   constexpr int stage = 32 * NW * Cfg<__bf16, D>::OROWV * 16;
   constexpr int smem = tiles > stage ? tiles : stage;
   auto kern = attn_fwd_bf16_kernel<D, JVP, NW>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
-      return -7;
-    attr_set = true;
-  }
+  static bool lds_ok[64] = {};
+  if (!ensure_dynamic_lds(kern, smem, lds_ok)) return -7;
   const uint32_t nqb = (p.Lq + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(64 * NW), smem, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : -7;

@@ -28,6 +28,20 @@ struct BwdParams {
   float scale, scale_log2;
 };
 
+// Opt a kernel in to `bytes` of dynamic LDS on the current device.  The attribute is per device, so the
+// "already done" flag is kept per (kernel instantiation, device); a race between two host threads at worst
+// repeats the idempotent call.
+template <typename K>
+inline bool ensure_dynamic_lds(K kernel, int bytes, bool (&done)[64]) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  if (!done[dev]) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+    done[dev] = true;
+  }
+  return true;
+}
+
 // Return 0 or a negative DMF_ATTN_E* code.
 int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream);
 // Building blocks of launch_fwd: the generic kernels (fp32 and bf16, any length)
