@@ -1,4 +1,4 @@
-"""ctypes binding of the C ABI declared in include/dmf_attn.h.
+"""ctypes binding of the C ABI declared in include/dmf_attn.h and include/dmf_block.h.
 
 The library is loaded from ``dmf_amd/libdmf_attn.so`` (built in-tree by
 ``python -m dmf_amd.build``).  There is deliberately no fallback: a missing
@@ -19,8 +19,8 @@ LIB_PATH = os.path.join(_HERE, "libdmf_attn.so")
 DMF_ATTN_F32, DMF_ATTN_BF16 = 0, 1
 SUPPORTED_HEAD_DIMS = (32, 64, 72, 80, 96, 128)
 
-# name -> (restype, argtypes): the complete exported surface of include/dmf_attn.h
-_P, _I, _F = c_void_p, c_int, c_float
+# name -> (restype, argtypes): the complete exported surface of include/dmf_attn.h and include/dmf_block.h
+_P, _I, _F, _L = c_void_p, c_int, c_float, c_int64
 _S = POINTER(c_int64)
 SIGNATURES = {
     "dmf_attn_version": (c_int, []),
@@ -28,6 +28,15 @@ SIGNATURES = {
     "dmf_attn_fwd_jvp": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_bwd": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
+    "dmf_block_workspace_floats": (c_int64, [_I] * 4),
+    "dmf_ln_modulate_fwd": (c_int, [_P] * 8 + [_S] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
+    "dmf_ln_modulate_bwd": (c_int, [_P] * 7 + [_L] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
+    "dmf_gate_residual_fwd": (c_int, [_P] * 8 + [_S] + [_I] * 3 + [_I] * 3 + [_P]),
+    "dmf_gate_residual_bwd": (c_int, [_P] * 6 + [_L] + [_I] * 3 + [_I] * 3 + [_P]),
+    "dmf_gelu_tanh_fwd": (c_int, [_P] * 4 + [_L, _I, _P]),
+    "dmf_gelu_tanh_bwd": (c_int, [_P] * 3 + [_L, _I, _P]),
+    "dmf_rmsnorm_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
+    "dmf_rmsnorm_bwd": (c_int, [_P] * 6 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
 }
 
 _lib = None
@@ -161,3 +170,180 @@ def bwd(dout, q, k, v, o, lse, scale: float):
             _strides(dout, q, k, v, o, dq, dk, dv), B, H, Lq, Lkv, D, float(scale), _dtype_code(q), _stream(q))
     _check(rc, "dmf_attn_bwd")
     return dq, dk, dv
+
+
+# ---- fused block glue (include/dmf_block.h) -----------------------------------------------------------------------
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _dense(t):
+    """Contiguous, functorch-unwrapped (None passes through)."""
+    if t is None:
+        return None
+    t = _raw(t)
+    return t if t.is_contiguous() else _raw(t.contiguous())
+
+
+def _mod(t, B: int, C: int):
+    """A per-sample modulation vector, (B, C) or (B, 1, C) with unit channel
+    stride -> (tensor, batch stride in elements); chunks of a wider adaLN output
+    are passed through without a copy."""
+    if t is None:
+        return None, 0
+    t = _raw(t)
+    if t.numel() != B * C or t.shape[0] != B or t.shape[-1] != C:
+        raise ValueError(f"expected a (B, C) or (B, 1, C) modulation tensor with B={B}, C={C}, got {tuple(t.shape)}")
+    eb = t.element_size()
+    if t.stride(-1) != 1 or t.data_ptr() % 16 or (t.stride(0) * eb) % 16:
+        t = _raw(t.contiguous())
+    return t, (t.stride(0) if B > 1 else C)
+
+
+def _same_dtype(what: str, *ts):
+    ts = [t for t in ts if t is not None]
+    for t in ts[1:]:
+        if t.dtype != ts[0].dtype or t.device != ts[0].device:
+            raise ValueError(f"{what}: operands must share dtype and device")
+
+
+def _blc(x):
+    if not x.is_cuda:
+        raise RuntimeError("dmf_amd block kernels run on the GPU only (tensor is on %s)" % x.device)
+    if x.dim() != 3:
+        raise ValueError(f"expected a (B, L, C) tensor, got shape {tuple(x.shape)}")
+    return x.shape
+
+
+def _workspace(which: int, B: int, L: int, dim: int, device) -> torch.Tensor:
+    n = load().dmf_block_workspace_floats(which, B, L, dim)
+    return _empty((max(int(n), 1),), torch.float32, device)
+
+
+def ln_modulate_fwd(x, shift, scale, tx=None, tshift=None, tscale=None, eps: float = 1e-6, out_dtype=None, jvp=False):
+    """(y, ty) of LayerNorm(x)*(1+scale)+shift; ty is None unless ``jvp``."""
+    B, L, C = _blc(x)
+    _same_dtype("ln_modulate x", x, tx)
+    _same_dtype("ln_modulate shift/scale", shift, scale, tshift, tscale)
+    x, tx = _dense(x), _dense(tx)
+    (shift, s0), (scale, s1), (tshift, s2), (tscale, s3) = (_mod(t, B, C) for t in (shift, scale, tshift, tscale))
+    out_dtype = out_dtype or x.dtype
+    y = _empty((B, L, C), out_dtype, x.device)
+    ty = _empty((B, L, C), out_dtype, x.device) if jvp else None
+    with torch.cuda.device(x.device):
+        rc = load().dmf_ln_modulate_fwd(
+            x.data_ptr(), _ptr(tx), shift.data_ptr(), scale.data_ptr(), _ptr(tshift), _ptr(tscale), y.data_ptr(), _ptr(ty),
+            (c_int64 * 4)(s0, s1, s2, s3), B, L, C, float(eps), _dtype_code(x), _dtype_code(shift), _dtype_code(y), _stream(x))
+    _check(rc, "dmf_ln_modulate_fwd")
+    return y, ty
+
+
+def ln_modulate_bwd(gy, x, scale, eps: float = 1e-6):
+    """(gx, gshift, gscale); gshift / gscale are dense (B, C) of scale's dtype."""
+    B, L, C = _blc(x)
+    gy, x = _dense(gy), _dense(x)
+    scale, ss = _mod(scale, B, C)
+    gx = _empty((B, L, C), x.dtype, x.device)
+    gshift = _empty((B, C), scale.dtype, x.device)
+    gscale = _empty((B, C), scale.dtype, x.device)
+    ws = _workspace(0, B, L, C, x.device)
+    with torch.cuda.device(x.device):
+        rc = load().dmf_ln_modulate_bwd(
+            gy.data_ptr(), x.data_ptr(), scale.data_ptr(), gx.data_ptr(), gshift.data_ptr(), gscale.data_ptr(), ws.data_ptr(),
+            ss, B, L, C, float(eps), _dtype_code(x), _dtype_code(scale), _dtype_code(gy), _stream(x))
+    _check(rc, "dmf_ln_modulate_bwd")
+    return gx, gshift, gscale
+
+
+def gate_residual_fwd(x, gate, h, tx=None, tgate=None, th=None, jvp=False):
+    """(y, ty) of x + gate*h, dtype of x; ty is None unless ``jvp``."""
+    B, L, C = _blc(x)
+    _same_dtype("gate_residual x", x, tx)
+    _same_dtype("gate_residual h", h, th)
+    _same_dtype("gate_residual gate", gate, tgate)
+    if h.shape != x.shape:
+        raise ValueError("gate_residual: x and h must have the same shape")
+    x, tx, h, th = _dense(x), _dense(tx), _dense(h), _dense(th)
+    (gate, g0), (tgate, g1) = _mod(gate, B, C), _mod(tgate, B, C)
+    y = _empty((B, L, C), x.dtype, x.device)
+    ty = _empty((B, L, C), x.dtype, x.device) if jvp else None
+    with torch.cuda.device(x.device):
+        rc = load().dmf_gate_residual_fwd(
+            x.data_ptr(), _ptr(tx), gate.data_ptr(), _ptr(tgate), h.data_ptr(), _ptr(th), y.data_ptr(), _ptr(ty),
+            (c_int64 * 2)(g0, g1), B, L, C, _dtype_code(x), _dtype_code(gate), _dtype_code(h), _stream(x))
+    _check(rc, "dmf_gate_residual_fwd")
+    return y, ty
+
+
+def gate_residual_bwd(gy, gate, h):
+    """(gh, ggate): gh like h, ggate dense (B, C) of gate's dtype."""
+    B, L, C = _blc(h)
+    gy, h = _dense(gy), _dense(h)
+    gate, gs = _mod(gate, B, C)
+    gh = _empty((B, L, C), h.dtype, h.device)
+    ggate = _empty((B, C), gate.dtype, h.device)
+    ws = _workspace(1, B, L, C, h.device)
+    with torch.cuda.device(h.device):
+        rc = load().dmf_gate_residual_bwd(
+            gy.data_ptr(), gate.data_ptr(), h.data_ptr(), gh.data_ptr(), ggate.data_ptr(), ws.data_ptr(),
+            gs, B, L, C, _dtype_code(gy), _dtype_code(gate), _dtype_code(h), _stream(h))
+    _check(rc, "dmf_gate_residual_bwd")
+    return gh, ggate
+
+
+def gelu_tanh_fwd(x, tx=None):
+    """(y, ty) of tanh-GELU; ty is None when ``tx`` is None."""
+    if not x.is_cuda:
+        raise RuntimeError("dmf_amd block kernels run on the GPU only (tensor is on %s)" % x.device)
+    _same_dtype("gelu_tanh", x, tx)
+    x, tx = _dense(x), _dense(tx)
+    y = _empty(x.shape, x.dtype, x.device)
+    ty = _empty(x.shape, x.dtype, x.device) if tx is not None else None
+    with torch.cuda.device(x.device):
+        rc = load().dmf_gelu_tanh_fwd(x.data_ptr(), _ptr(tx), y.data_ptr(), _ptr(ty), x.numel(), _dtype_code(x), _stream(x))
+    _check(rc, "dmf_gelu_tanh_fwd")
+    return y, ty
+
+
+def gelu_tanh_bwd(gy, x):
+    _same_dtype("gelu_tanh_bwd", x, gy)
+    gy, x = _dense(gy), _dense(x)
+    gx = _empty(x.shape, x.dtype, x.device)
+    with torch.cuda.device(x.device):
+        rc = load().dmf_gelu_tanh_bwd(gy.data_ptr(), x.data_ptr(), gx.data_ptr(), x.numel(), _dtype_code(x), _stream(x))
+    _check(rc, "dmf_gelu_tanh_bwd")
+    return gx
+
+
+def rmsnorm_fwd(x, gain, tx=None, eps: float = 1e-6, jvp=False):
+    """(y, ty) of the per-head RMS norm of a (B, L, H, D) tensor (strided views are
+    read in place); outputs are contiguous."""
+    _check_inputs(x, *([tx] if tx is not None else []))
+    x, tx = _prep(x), (None if tx is None else _prep(tx))
+    gain = _dense(gain)
+    B, L, H, D = x.shape
+    y = _empty((B, L, H, D), x.dtype, x.device)
+    ty = _empty((B, L, H, D), x.dtype, x.device) if jvp else None
+    with torch.cuda.device(x.device):
+        rc = load().dmf_rmsnorm_fwd(
+            x.data_ptr(), _ptr(tx), gain.data_ptr(), y.data_ptr(), _ptr(ty), _strides(x, tx if tx is not None else x),
+            B, L, H, D, float(eps), _dtype_code(x), _dtype_code(gain), _stream(x))
+    _check(rc, "dmf_rmsnorm_fwd")
+    return y, ty
+
+
+def rmsnorm_bwd(gy, x, gain, eps: float = 1e-6):
+    """(gx, ggain): gx contiguous (B, L, H, D), ggain (D) of gain's dtype."""
+    _check_inputs(x, gy)
+    x, gy, gain = _prep(x), _dense(gy), _dense(gain)
+    B, L, H, D = x.shape
+    gx = _empty((B, L, H, D), x.dtype, x.device)
+    ggain = _empty((D,), gain.dtype, x.device)
+    ws = _workspace(2, B, L, D, x.device)
+    with torch.cuda.device(x.device):
+        rc = load().dmf_rmsnorm_bwd(
+            gy.data_ptr(), x.data_ptr(), gain.data_ptr(), gx.data_ptr(), ggain.data_ptr(), ws.data_ptr(), _strides(x),
+            B, L, H, D, float(eps), _dtype_code(x), _dtype_code(gain), _stream(x))
+    _check(rc, "dmf_rmsnorm_bwd")
+    return gx, ggain

@@ -1,0 +1,172 @@
+"""Fused DiT-block glue operators with forward-mode (JVP) support.
+
+Host-side counterparts of the small tensor expressions that surround the
+attention operator in the reference's block (models/layers.py):
+
+* ``ln_modulate(x, shift, scale)``  = ``modulate(LayerNorm(x), shift, scale)``   (:28-29, :198, :200, :219)
+* ``gate_residual(x, gate, h)``     = ``x + gate * h``                           (:198, :200)
+* ``gelu_tanh(x)``                  = ``nn.GELU(approximate="tanh")(x)``         (:162, :166)
+* ``rms_norm(x, gain)``             = ``RMSNorm.forward``                        (:33-42, :148)
+
+Each follows the protocol of the attention operator (flash_attention_hip_jvp):
+a wrapper unpacks forward-AD duals, one ``torch.autograd.Function`` call pushes
+primal and tangent through a single fused kernel (C ABI: include/dmf_block.h),
+and the result is re-packed with ``fwAD.make_dual``.  ``backward`` propagates
+through the primal output only: tangent inputs get no gradient and the
+cotangent of the tangent output is dropped -- exact for the MeanFlow loss, whose
+JVP target is detached (loss.py:171-172), and the same convention as the
+reference's attention ``backward`` (flash_attention_2_jvp.py:260-276).
+There is no fallback: without the HIP library every call raises.
+"""
+from __future__ import annotations
+
+import torch
+import torch.autograd.forward_ad as fwAD
+
+from . import _lib
+
+
+def _unpack(*tensors):
+    primals, tangents = [], []
+    for t in tensors:
+        p, tg = fwAD.unpack_dual(t)
+        primals.append(p)
+        tangents.append(tg)
+    return primals, tangents, any(tg is not None for tg in tangents)
+
+
+def _like(g, ref):
+    """Gradient of a (B, C) modulation operand reshaped to the operand's shape."""
+    return g.reshape(ref)
+
+
+class LNModulateFunc(torch.autograd.Function):
+    """(x, shift, scale, tx, tshift, tscale, eps, out_dtype, jvp) -> (y, ty)."""
+
+    @staticmethod
+    def forward(x, shift, scale, tx, tshift, tscale, eps, out_dtype, jvp):
+        return _lib.ln_modulate_fwd(x, shift, scale, tx, tshift, tscale, eps, out_dtype, jvp)
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        x, shift, scale, _, _, _, eps, _, _ = inputs
+        ctx.save_for_backward(x, scale)
+        ctx.eps, ctx.mod_shape = eps, (shift.shape, scale.shape)
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, gy, gty):
+        if gy is None:
+            return (None,) * 9
+        x, scale = ctx.saved_tensors
+        gx, gshift, gscale = _lib.ln_modulate_bwd(gy, x, scale, ctx.eps)
+        return gx, _like(gshift, ctx.mod_shape[0]), _like(gscale, ctx.mod_shape[1]), None, None, None, None, None, None
+
+
+class GateResidualFunc(torch.autograd.Function):
+    """(x, gate, h, tx, tgate, th, jvp) -> (y, ty)."""
+
+    @staticmethod
+    def forward(x, gate, h, tx, tgate, th, jvp):
+        return _lib.gate_residual_fwd(x, gate, h, tx, tgate, th, jvp)
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        x, gate, h = inputs[:3]
+        ctx.save_for_backward(gate, h)
+        ctx.gate_shape, ctx.x_dtype = gate.shape, x.dtype
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, gy, gty):
+        if gy is None:
+            return (None,) * 7
+        gate, h = ctx.saved_tensors
+        gh, ggate = _lib.gate_residual_bwd(gy, gate, h)
+        return gy, _like(ggate, ctx.gate_shape), gh, None, None, None, None
+
+
+class GeluTanhFunc(torch.autograd.Function):
+    """(x, tx) -> (y, ty)."""
+
+    @staticmethod
+    def forward(x, tx):
+        return _lib.gelu_tanh_fwd(x, tx)
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        ctx.save_for_backward(inputs[0])
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, gy, gty):
+        if gy is None:
+            return None, None
+        (x,) = ctx.saved_tensors
+        return _lib.gelu_tanh_bwd(gy.to(x.dtype), x), None
+
+
+class RMSNormFunc(torch.autograd.Function):
+    """(x, gain, tx, eps, jvp) -> (y, ty); x is (B, L, H, D), normalised over D."""
+
+    @staticmethod
+    def forward(x, gain, tx, eps, jvp):
+        return _lib.rmsnorm_fwd(x, gain, tx, eps, jvp)
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        x, gain, _, eps, _ = inputs
+        ctx.save_for_backward(x, gain)
+        ctx.eps = eps
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, gy, gty):
+        if gy is None:
+            return (None,) * 5
+        x, gain = ctx.saved_tensors
+        gx, ggain = _lib.rmsnorm_bwd(gy.to(x.dtype), x, gain, ctx.eps)
+        return gx, ggain, None, None, None
+
+
+def _autocast_dtype(x: torch.Tensor):
+    if x.is_cuda and torch.is_autocast_enabled("cuda"):
+        return torch.get_autocast_dtype("cuda")
+    return x.dtype
+
+
+def ln_modulate(x, shift, scale, eps: float = 1e-6):
+    """``LayerNorm(x) * (1 + scale) + shift`` for x (B, L, C) and shift / scale
+    (B, C) or (B, 1, C); LayerNorm over C without affine parameters.  Under
+    autocast the result is produced directly in the autocast dtype (it only ever
+    feeds a Linear, which would cast it)."""
+    (xp, shp, scp), (tx, tsh, tsc), dual = _unpack(x, shift, scale)
+    y, ty = LNModulateFunc.apply(xp, shp, scp, tx, tsh, tsc, eps, _autocast_dtype(xp), dual)
+    return fwAD.make_dual(y, ty) if dual else y
+
+
+def gate_residual(x, gate, h):
+    """``x + gate * h`` for x, h (B, L, C) and gate (B, C) or (B, 1, C); the result
+    has the promoted dtype of x and h (the fp32 residual stream under autocast)."""
+    (xp, gp, hp), (tx, tg, th), dual = _unpack(x, gate, h)
+    dt = torch.promote_types(xp.dtype, hp.dtype)
+    if xp.dtype != dt:
+        xp, tx = xp.to(dt), (None if tx is None else tx.to(dt))
+    y, ty = GateResidualFunc.apply(xp, gp, hp, tx, tg, th, dual)
+    return fwAD.make_dual(y, ty) if dual else y
+
+
+def gelu_tanh(x):
+    """tanh-approximated GELU."""
+    (xp,), (tx,), dual = _unpack(x)
+    y, ty = GeluTanhFunc.apply(xp, tx)
+    return fwAD.make_dual(y, ty) if dual else y
+
+
+def rms_norm(x, gain, eps: float = 1e-6):
+    """Per-head RMS norm of a (B, L, H, D) tensor over D (strided views into a
+    packed qkv buffer are read in place); returns a contiguous tensor.  The gain
+    is treated as a constant by forward-mode AD (parameters carry no tangent)."""
+    (xp,), (tx,), dual = _unpack(x)
+    y, ty = RMSNormFunc.apply(xp, gain, tx, eps, dual)
+    return fwAD.make_dual(y, ty) if dual else y

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdmf_attn.so")
 PROBE_LIB = os.path.join(HERE, "libdmf_probe.so")
-SOURCES = ["attn_fwd.hip", "attn_fwd_bf16.hip", "attn_bwd.hip", "attn_bwd_bf16.hip", "dmf_attn_abi.hip"]
+SOURCES = ["attn_fwd.hip", "attn_fwd_bf16.hip", "attn_bwd.hip", "attn_bwd_bf16.hip", "dmf_attn_abi.hip", "block_ops.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

@@ -1,0 +1,131 @@
+/*
+ * dmf_block.h -- C ABI of the fused transformer-block glue kernels (gfx950)
+ * that sit either side of the attention operator in a DiT block, each with an
+ * optional forward-mode tangent stream computed in the same pass.
+ *
+ * Under `torch.func.jvp` (loss.py:165-170) the reference runs these pieces as
+ * strings of separate primal + tangent elementwise / reduction kernels:
+ *   - `modulate(norm(x), shift, scale)`   models/layers.py:28-29, 198, 200, 218-219
+ *   - `x + gate * branch`                  models/layers.py:198, 200
+ *   - `GELU(approximate="tanh")`           models/layers.py:162
+ *   - `RMSNorm` on q and k                 models/layers.py:33-42, 148
+ * Every entry point below replaces one such string by a single HBM pass.
+ *
+ * Conventions
+ *   - (B, L, C) activations are dense and row-major; per-sample modulation
+ *     vectors (shift / scale / gate and their tangents) are (B, C) with unit
+ *     channel stride and a caller-given batch stride in elements (they are
+ *     chunks of one (B, 6C) adaLN output, models/layers.py:197).
+ *   - dtype codes, return codes and `dmf_attn_strerror` are those of
+ *     dmf_attn.h.  All arithmetic is fp32; results are rounded once on store.
+ *   - A NULL tangent *input* means "zero tangent".  A NULL tangent *output*
+ *     selects the primal-only kernel.
+ *   - C (and the head dim D of the RMSNorm entry points) must be a multiple of
+ *     8; C <= 2048, D <= 128; base pointers and batch strides must keep every
+ *     row 16-byte aligned.
+ *   - The caller owns all memory (including the fp32 `workspace` of the
+ *     backward entry points, sized by dmf_block_workspace_floats); launches are
+ *     asynchronous on `stream` (hipStream_t as void*, NULL = default stream);
+ *     entry points are re-entrant.  The backward reductions are two-stage sums
+ *     in a fixed order (no atomics): results are run-to-run deterministic.
+ */
+#ifndef DMF_BLOCK_H
+#define DMF_BLOCK_H
+
+#include "dmf_attn.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Number of fp32 workspace elements a backward entry point needs.
+ * `which`: 0 = dmf_ln_modulate_bwd, 1 = dmf_gate_residual_bwd (rows = B*L, dim = C),
+ *          2 = dmf_rmsnorm_bwd (rows = B*L*H, dim = D).  Returns 0 on bad input. */
+DMF_ATTN_API int64_t dmf_block_workspace_floats(int which, int B, int L, int dim);
+
+/*
+ * y = LayerNorm(x) * (1 + scale) + shift, LayerNorm over C without affine
+ * parameters (biased variance, `eps` inside the square root), and -- when `ty`
+ * is given -- its tangent along (tx, tshift, tscale):
+ *   xh = (x - mean) * rstd,  dxh = rstd * (tx - mean(tx) - xh * mean(xh * tx)),
+ *   ty = dxh * (1 + scale) + xh * tscale + tshift.
+ * Replaces `modulate(self.norm1(x), shift_msa, scale_msa)` and its norm2 /
+ * norm_final twins (models/layers.py:198, 200, 219).
+ * x, tx: (B, L, C) of x_dtype.  shift, scale, tshift, tscale: (B, C) of
+ * mod_dtype with batch strides mod_strides[0..3] (in that order).  y, ty:
+ * (B, L, C) of y_dtype.
+ */
+DMF_ATTN_API int dmf_ln_modulate_fwd(const void* x, const void* tx, const void* shift, const void* scale,
+                                     const void* tshift, const void* tscale, void* y, void* ty,
+                                     const int64_t* mod_strides, int B, int L, int C, float eps,
+                                     int x_dtype, int mod_dtype, int y_dtype, void* stream);
+
+/*
+ * Backward of the primal of dmf_ln_modulate_fwd: given gy = dLoss/dy,
+ *   gx     = rstd * (g - mean(g) - xh * mean(g * xh)),  g = gy * (1 + scale)
+ *   gshift = sum_l gy,   gscale = sum_l gy * xh.
+ * gx: (B, L, C) of x_dtype; gshift, gscale: dense (B, C) of mod_dtype.
+ */
+DMF_ATTN_API int dmf_ln_modulate_bwd(const void* gy, const void* x, const void* scale, void* gx, void* gshift,
+                                     void* gscale, float* workspace, int64_t scale_stride, int B, int L, int C,
+                                     float eps, int x_dtype, int mod_dtype, int gy_dtype, void* stream);
+
+/*
+ * y = x + gate * h and, when `ty` is given, ty = tx + tgate * h + gate * th.
+ * Replaces `x + gate_msa * self.attn(...)` / `x + gate_mlp * self.mlp(...)`
+ * (models/layers.py:198, 200).  x, tx, y, ty: (B, L, C) of x_dtype; h, th:
+ * (B, L, C) of h_dtype; gate, tgate: (B, C) of mod_dtype with batch strides
+ * gate_strides[0..1].
+ */
+DMF_ATTN_API int dmf_gate_residual_fwd(const void* x, const void* tx, const void* gate, const void* tgate,
+                                       const void* h, const void* th, void* y, void* ty,
+                                       const int64_t* gate_strides, int B, int L, int C,
+                                       int x_dtype, int mod_dtype, int h_dtype, void* stream);
+
+/*
+ * Backward of the primal of dmf_gate_residual_fwd (dLoss/dx is gy itself and
+ * needs no kernel): gh = gate * gy ((B, L, C) of h_dtype), ggate = sum_l gy * h
+ * (dense (B, C) of mod_dtype).  gy: (B, L, C) of gy_dtype.
+ */
+DMF_ATTN_API int dmf_gate_residual_bwd(const void* gy, const void* gate, const void* h, void* gh, void* ggate,
+                                       float* workspace, int64_t gate_stride, int B, int L, int C,
+                                       int gy_dtype, int mod_dtype, int h_dtype, void* stream);
+
+/*
+ * y = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) over n elements and,
+ * when `ty` is given, ty = gelu'(x) * tx.  Replaces `self.act(...)` of the MLP
+ * (models/layers.py:162, 166).  n must be a multiple of 8.
+ */
+DMF_ATTN_API int dmf_gelu_tanh_fwd(const void* x, const void* tx, void* y, void* ty, int64_t n, int dtype,
+                                   void* stream);
+
+/* gx = gelu'(x) * gy over n elements (n a multiple of 8). */
+DMF_ATTN_API int dmf_gelu_tanh_bwd(const void* gy, const void* x, void* gx, int64_t n, int dtype, void* stream);
+
+/*
+ * Per-head RMS norm over D of a logical (B, L, H, D) tensor:
+ *   r = rsqrt(mean(x^2) + eps),  y = x * r * gain,
+ *   ty = (tx * r + x * dr) * gain,  dr = -r^3 * mean(x * tx)   (when `ty` is given).
+ * Replaces `self.q_norm(q)` / `self.k_norm(k)` (models/layers.py:33-42, 148).
+ * x and tx carry four element strides each ({sB, sL, sH, 1}; views into a
+ * packed qkv buffer qualify, models/layers.py:143-147): strides = {x[4], tx[4]}.
+ * y, ty: dense (B, L, H, D) of `dtype`.  gain: (D) of gain_dtype.
+ */
+DMF_ATTN_API int dmf_rmsnorm_fwd(const void* x, const void* tx, const void* gain, void* y, void* ty,
+                                 const int64_t* strides, int B, int L, int H, int D, float eps,
+                                 int dtype, int gain_dtype, void* stream);
+
+/*
+ * Backward of the primal of dmf_rmsnorm_fwd:
+ *   g = gy * gain,  gx = r * g - x * r^3 * mean(x * g),  ggain = sum_rows gy * x * r.
+ * x: strided as above (strides = {x[4]}); gy, gx: dense (B, L, H, D); ggain: (D)
+ * of gain_dtype.
+ */
+DMF_ATTN_API int dmf_rmsnorm_bwd(const void* gy, const void* x, const void* gain, void* gx, void* ggain,
+                                 float* workspace, const int64_t* strides, int B, int L, int H, int D, float eps,
+                                 int dtype, int gain_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DMF_BLOCK_H */

@@ -1,0 +1,181 @@
+"""GPU parity of the fused block-glue kernels (C ABI include/dmf_block.h) against
+the CPU oracle (oracle/block_oracle.py) on the same seeded inputs.
+
+Tolerances (relative L2): 1e-5 when everything is fp32; 6e-3 when the result is
+stored in bf16 (one rounding of an fp32 result, 2^-9 relative per element, so
+about 2.3e-3 in L2).  The oracle is always evaluated in fp32 on the values the
+kernel was given (bf16 inputs are rounded first, then widened)."""
+import pytest
+import torch
+
+from dmf_amd import _lib, block_ops
+from oracle import attn_oracle as ao
+from oracle import block_oracle as bo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+def _tol(*dtypes):
+    return 6e-3 if any(d == BF16 for d in dtypes) else 1e-5
+
+
+def _close(got, ref, tol, what=""):
+    err = ao.rel_l2(got.float().cpu(), ref.float())
+    assert err <= tol, f"{what}: rel-L2 {err:.3e} > {tol:.1e}"
+
+
+def _rounded(d, keys, dtype):
+    """Round the named inputs to dtype (what the kernel sees) and return fp32 CPU copies + device copies."""
+    cpu = {k: d[k].to(dtype).float() for k in keys}
+    dev = {k: d[k].to(dtype).to(DEV) for k in keys}
+    return cpu, dev
+
+
+SHAPES = [(2, 37, 768), (3, 64, 1152), (1, 5, 8), (2, 33, 2048), (2, 16, 1024), (4, 1, 384)]
+DTYPES = [(F32, F32, F32), (F32, BF16, BF16), (BF16, BF16, BF16)]   # (x, mods, out)
+
+
+@pytest.mark.parametrize("B,L,C", SHAPES)
+@pytest.mark.parametrize("xdt,mdt,ydt", DTYPES)
+def test_ln_modulate_fwd_jvp_bwd(B, L, C, xdt, mdt, ydt):
+    print(f"ln_modulate B{B} L{L} C{C} {xdt} {mdt} {ydt}", flush=True)
+    d = bo.make_block_inputs(B, L, C, seed=11)
+    cx, gx_ = _rounded(d, ("x", "tx"), xdt)
+    cm, gm = _rounded(d, ("shift", "scale", "tshift", "tscale"), mdt)
+    cg, gg = _rounded(d, ("gy",), ydt)
+    y_ref, ty_ref = bo.jvp(bo.ln_modulate, (cx["x"], cm["shift"], cm["scale"]), (cx["tx"], cm["tshift"], cm["tscale"]))
+    tol = _tol(xdt, mdt, ydt)
+    y, ty = _lib.ln_modulate_fwd(gx_["x"], gm["shift"], gm["scale"], gx_["tx"], gm["tshift"], gm["tscale"], 1e-6, ydt, True)
+    assert y.dtype == ydt and ty.dtype == ydt
+    _close(y, y_ref, tol, "y")
+    _close(ty, ty_ref, tol, "ty")
+    y0, none = _lib.ln_modulate_fwd(gx_["x"], gm["shift"], gm["scale"], eps=1e-6, out_dtype=ydt)
+    assert none is None and torch.equal(y0, y)
+    # missing tangents read as zeros
+    _, ty_x = _lib.ln_modulate_fwd(gx_["x"], gm["shift"], gm["scale"], gx_["tx"], None, None, 1e-6, ydt, True)
+    z = torch.zeros_like(cm["shift"])
+    _, ty_x_ref = bo.jvp(bo.ln_modulate, (cx["x"], cm["shift"], cm["scale"]), (cx["tx"], z, z))
+    _close(ty_x, ty_x_ref, tol, "ty (x tangent only)")
+    gx_ref, gsh_ref, gsc_ref = bo.grads(bo.ln_modulate, (cx["x"], cm["shift"], cm["scale"]), cg["gy"])
+    gx, gsh, gsc = _lib.ln_modulate_bwd(gg["gy"], gx_["x"], gm["scale"], 1e-6)
+    assert gx.dtype == xdt and gsh.dtype == mdt and gsh.shape == (B, C)
+    _close(gx, gx_ref, _tol(xdt, ydt), "gx")
+    _close(gsh.view(B, 1, C), gsh_ref, _tol(mdt), "gshift")
+    _close(gsc.view(B, 1, C), gsc_ref, _tol(mdt), "gscale")
+
+
+@pytest.mark.parametrize("B,L,C", SHAPES)
+@pytest.mark.parametrize("xdt,mdt,hdt", DTYPES)
+def test_gate_residual_fwd_jvp_bwd(B, L, C, xdt, mdt, hdt):
+    print(f"gate_residual B{B} L{L} C{C} {xdt} {mdt} {hdt}", flush=True)
+    d = bo.make_block_inputs(B, L, C, seed=12)
+    cx, gx_ = _rounded(d, ("x", "tx", "gy"), xdt)
+    cm, gm = _rounded(d, ("gate", "tgate"), mdt)
+    ch, gh_ = _rounded(d, ("h", "th"), hdt)
+    y_ref, ty_ref = bo.jvp(bo.gate_residual, (cx["x"], cm["gate"], ch["h"]), (cx["tx"], cm["tgate"], ch["th"]))
+    y, ty = _lib.gate_residual_fwd(gx_["x"], gm["gate"], gh_["h"], gx_["tx"], gm["tgate"], gh_["th"], True)
+    assert y.dtype == xdt
+    _close(y, y_ref, _tol(xdt), "y")
+    _close(ty, ty_ref, _tol(xdt), "ty")
+    y0, none = _lib.gate_residual_fwd(gx_["x"], gm["gate"], gh_["h"])
+    assert none is None and torch.equal(y0, y)
+    _, gg_ref, gh_ref = bo.grads(bo.gate_residual, (cx["x"], cm["gate"], ch["h"]), cx["gy"])
+    gh, gg = _lib.gate_residual_bwd(gx_["gy"], gm["gate"], gh_["h"])
+    _close(gh, gh_ref, _tol(hdt), "gh")
+    _close(gg.view(B, 1, C), gg_ref, _tol(mdt), "ggate")
+
+
+@pytest.mark.parametrize("shape", [(2, 37, 3072), (1, 8), (3, 5, 4608)])
+@pytest.mark.parametrize("dt", [F32, BF16])
+def test_gelu_tanh_fwd_jvp_bwd(shape, dt):
+    print(f"gelu {shape} {dt}", flush=True)
+    g = torch.Generator().manual_seed(13)
+    x, t = (2 * torch.randn(*shape, generator=g)).to(dt), torch.randn(*shape, generator=g).to(dt)
+    y_ref, ty_ref = bo.jvp(bo.gelu_tanh, (x.float(),), (t.float(),))
+    y, ty = _lib.gelu_tanh_fwd(x.to(DEV), t.to(DEV))
+    _close(y, y_ref, _tol(dt), "y")
+    _close(ty, ty_ref, _tol(dt), "ty")
+    y0, none = _lib.gelu_tanh_fwd(x.to(DEV))
+    assert none is None and torch.equal(y0, y)
+    (gx_ref,) = bo.grads(bo.gelu_tanh, (x.float(),), t.float())
+    _close(_lib.gelu_tanh_bwd(t.to(DEV), x.to(DEV)), gx_ref, _tol(dt), "gx")
+
+
+@pytest.mark.parametrize("B,L,H,D", [(2, 37, 16, 72), (1, 5, 3, 64), (2, 9, 2, 128), (1, 300, 5, 8), (2, 64, 12, 96)])
+@pytest.mark.parametrize("dt", [F32, BF16])
+@pytest.mark.parametrize("packed", [False, True])
+def test_rmsnorm_fwd_jvp_bwd(B, L, H, D, dt, packed):
+    print(f"rmsnorm B{B} L{L} H{H} D{D} {dt} packed={packed}", flush=True)
+    g = torch.Generator().manual_seed(14)
+    x, tx, gy = (torch.randn(B, L, H, D, generator=g).to(dt) for _ in range(3))
+    gain = 1 + 0.2 * torch.randn(D, generator=g)
+
+    def dev(t):
+        if not packed:
+            return t.to(DEV)
+        buf = torch.zeros(B, L, 3, H, D, dtype=dt, device=DEV)   # q-slot view of a packed qkv buffer
+        buf[:, :, 0] = t.to(DEV)
+        return buf[:, :, 0]
+
+    cf = bo.rms_norm_closed_fp64(x.float(), gain, tx.float(), gy.float())
+    y, ty = _lib.rmsnorm_fwd(dev(x), gain.to(DEV), dev(tx), 1e-6, True)
+    assert y.is_contiguous() and y.dtype == dt
+    _close(y, torch.from_numpy(cf["y"]), _tol(dt), "y")
+    _close(ty, torch.from_numpy(cf["ty"]), _tol(dt), "ty")
+    if dt == F32:  # the reference's own rounding points only matter in bf16; in fp32 the restatement agrees too
+        _close(y, bo.rms_norm(x, gain), 1e-5, "y vs restated RMSNorm.forward")
+    y0, none = _lib.rmsnorm_fwd(dev(x), gain.to(DEV))
+    assert none is None and torch.equal(y0, y)
+    gx, ggain = _lib.rmsnorm_bwd(gy.to(DEV), dev(x), gain.to(DEV))
+    _close(gx, torch.from_numpy(cf["gx"]), _tol(dt), "gx")
+    _close(ggain, torch.from_numpy(cf["ggain"]), 1e-5, "ggain")
+
+
+def test_wrappers_under_func_jvp_and_autograd():
+    """The dual-aware wrappers under torch.func.jvp with autograd on top, as the training step uses them."""
+    B, L, C = 2, 24, 384
+    d = bo.make_block_inputs(B, L, C, seed=15)
+    dev = {k: v.to(DEV) for k, v in d.items()}
+
+    def fused(x, shift, scale, gate):
+        return block_ops.gate_residual(x, gate, block_ops.gelu_tanh(block_ops.ln_modulate(x, shift, scale)))
+
+    def plain(x, shift, scale, gate):
+        return bo.gate_residual(x, gate, bo.gelu_tanh(bo.ln_modulate(x, shift, scale)))
+
+    keys, tkeys = ("x", "shift", "scale", "gate"), ("tx", "tshift", "tscale", "tgate")
+    prim = [dev[k].clone().requires_grad_(True) for k in keys]
+    y, ty = torch.func.jvp(fused, tuple(prim), tuple(dev[k] for k in tkeys))
+    y_ref, ty_ref = bo.jvp(plain, [d[k] for k in keys], [d[k] for k in tkeys])
+    _close(y, y_ref, 1e-5, "y")
+    _close(ty, ty_ref, 1e-5, "ty")
+    (y * dev["gy"]).sum().backward()
+    refs = bo.grads(plain, [d[k] for k in keys], d["gy"])
+    for k, p, r in zip(keys, prim, refs):
+        _close(p.grad, r, 2e-5, f"grad {k}")
+    # plain (non-dual) call gives the same primal
+    assert torch.allclose(fused(*[dev[k] for k in keys]), y.detach(), atol=0, rtol=0)
+
+
+def test_rms_norm_wrapper_under_func_jvp():
+    g = torch.Generator().manual_seed(16)
+    x, tx = torch.randn(2, 20, 4, 72, generator=g), torch.randn(2, 20, 4, 72, generator=g)
+    gain = (1 + 0.2 * torch.randn(72, generator=g))
+    y, ty = torch.func.jvp(lambda a: block_ops.rms_norm(a, gain.to(DEV)), (x.to(DEV),), (tx.to(DEV),))
+    cf = bo.rms_norm_closed_fp64(x, gain, tx)
+    _close(y, torch.from_numpy(cf["y"]), 1e-5)
+    _close(ty, torch.from_numpy(cf["ty"]), 1e-5)
+
+
+def test_block_abi_rejects_bad_arguments():
+    x = torch.zeros(2, 4, 20, device=DEV)        # C = 20 is not a multiple of 8
+    m = torch.zeros(2, 20, device=DEV)
+    with pytest.raises(RuntimeError, match="bad shape"):
+        _lib.ln_modulate_fwd(x, m, m)
+    big = torch.zeros(1, 2, 4096, device=DEV)    # C above the supported maximum
+    with pytest.raises(RuntimeError, match="bad shape"):
+        _lib.gate_residual_fwd(big, torch.zeros(1, 4096, device=DEV), big)
+    with pytest.raises(RuntimeError, match="head dim"):
+        _lib.rmsnorm_fwd(torch.zeros(1, 2, 2, 20, device=DEV), torch.ones(20, device=DEV))
