@@ -37,6 +37,7 @@ SIGNATURES = {
     "dmf_gelu_tanh_bwd": (c_int, [_P] * 3 + [_L, _I, _P]),
     "dmf_rmsnorm_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_rmsnorm_bwd": (c_int, [_P] * 6 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
+    "dmf_colsum": (c_int, [_P] * 3 + [_L, _I, _I, _I, _P]),
 }
 
 _lib = None
@@ -347,3 +348,20 @@ def rmsnorm_bwd(gy, x, gain, eps: float = 1e-6):
             B, L, H, D, float(eps), _dtype_code(x), _dtype_code(gain), _stream(x))
     _check(rc, "dmf_rmsnorm_bwd")
     return gx, ggain
+
+
+def colsum(x, out_dtype=None):
+    """Column sums of a dense 2-D tensor (rows, C) -> (C,), fixed summation order."""
+    if not x.is_cuda:
+        raise RuntimeError("dmf_amd block kernels run on the GPU only (tensor is on %s)" % x.device)
+    if x.dim() != 2:
+        raise ValueError(f"expected a (rows, C) matrix, got shape {tuple(x.shape)}")
+    x = _dense(x)
+    rows, C = x.shape
+    out = _empty((C,), out_dtype or x.dtype, x.device)
+    n = load().dmf_block_workspace_floats(3, 1, min(rows, 2 ** 31 - 1), C)
+    ws = _empty((max(int(n), 1),), torch.float32, x.device)
+    with torch.cuda.device(x.device):
+        rc = load().dmf_colsum(x.data_ptr(), out.data_ptr(), ws.data_ptr(), rows, C, _dtype_code(x), _dtype_code(out), _stream(x))
+    _check(rc, "dmf_colsum")
+    return out

@@ -7,6 +7,7 @@ attention operator in the reference's block (models/layers.py):
 * ``gate_residual(x, gate, h)``     = ``x + gate * h``                           (:198, :200)
 * ``gelu_tanh(x)``                  = ``nn.GELU(approximate="tanh")(x)``         (:162, :166)
 * ``rms_norm(x, gain)``             = ``RMSNorm.forward``                        (:33-42, :148)
+* ``dual_linear(x, weight, bias)``  = ``nn.Linear`` (:131,137,161-165,...) -- library GEMMs, see ``DualLinearFunc``
 
 Each follows the protocol of the attention operator (flash_attention_hip_jvp):
 a wrapper unpacks forward-AD duals, one ``torch.autograd.Function`` call pushes
@@ -127,6 +128,52 @@ class RMSNormFunc(torch.autograd.Function):
         x, gain = ctx.saved_tensors
         gx, ggain = _lib.rmsnorm_bwd(gy.to(x.dtype), x, gain, ctx.eps)
         return gx, ggain, None, None, None
+
+
+class DualLinearFunc(torch.autograd.Function):
+    """(x, tx, weight, bias) -> (y, ty) = (x W^T + b, tx W^T): exactly one library
+    GEMM per stream.  torch's own forward-mode rule for ``linear`` also multiplies
+    the primal input by a materialised all-zero weight tangent and adds the two
+    products (three GEMMs, two fills, a copy and an add per layer); parameters
+    carry no tangent in the MeanFlow JVP (loss.py:165-170), so that work is
+    skipped here.  Runs under autocast like ``F.linear``."""
+
+    @staticmethod
+    def forward(x, tx, weight, bias):
+        y = torch.nn.functional.linear(x, weight, bias)
+        ty = None if tx is None else torch.nn.functional.linear(tx, weight)
+        return y, ty
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        x, _, weight, bias = inputs
+        ctx.save_for_backward(x, weight)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, gy, gty):
+        if gy is None:
+            return None, None, None, None
+        x, weight = ctx.saved_tensors
+        g2 = gy.reshape(-1, gy.shape[-1])
+        x2 = x.reshape(-1, x.shape[-1]).to(g2.dtype)
+        gx = (g2 @ weight.to(g2.dtype)).reshape(x.shape).to(x.dtype) if ctx.needs_input_grad[0] else None
+        gw = (g2.t() @ x2).to(weight.dtype) if ctx.needs_input_grad[2] else None
+        gb = None
+        if ctx.bias_dtype is not None and ctx.needs_input_grad[3]:
+            # torch's multi-block column reduction clears its scratch with a memset node, which does not survive
+            # HIP-graph replay; the library's two-stage sum has no such node
+            gb = _lib.colsum(g2.contiguous(), ctx.bias_dtype) if g2.is_cuda and g2.shape[1] % 8 == 0 else g2.sum(0).to(ctx.bias_dtype)
+        return gx, None, gw, gb
+
+
+def dual_linear(x, weight, bias=None):
+    """``F.linear(x, weight, bias)``; a forward-AD dual ``x`` gives a dual result
+    (weight and bias are constants of the tangent map)."""
+    (xp,), (tx,), dual = _unpack(x)
+    y, ty = DualLinearFunc.apply(xp, tx, weight, bias)
+    return fwAD.make_dual(y, ty) if dual else y
 
 
 def _autocast_dtype(x: torch.Tensor):

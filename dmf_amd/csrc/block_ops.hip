@@ -308,6 +308,7 @@ __global__ __launch_bounds__(kThreads) void reduce_partials_kernel(ReduceParams 
   const int64_t b = bk / p.K;
   float s[8];
   zero8(s);
+#pragma unroll 8
   for (int c = 0; c < p.nchunk; ++c) {
     float t[8];
     load8(p.partial, 0, ((b * p.nchunk + c) * p.K + k) * p.C + col, t);
@@ -543,6 +544,35 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(RmsParams p) {
   }
 }
 
+// ---- column sums of a dense (rows, C) matrix ----------------------------------------------------------------------
+// Work-group (x, y): rows [x*kColsumRows, +kColsumRows), vector columns y*kThreads + thread.
+
+constexpr int kColsumRows = 64;
+
+struct ColsumParams {
+  const void* x;
+  float* partial;  // (nchunk, C)
+  int64_t rows;
+  int C;
+  int xbf;
+};
+
+__global__ __launch_bounds__(kThreads) void colsum_kernel(ColsumParams p) {
+  const int col = (blockIdx.y * kThreads + threadIdx.x) * 8;
+  if (col >= p.C) return;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kColsumRows;
+  const int64_t r1 = r0 + kColsumRows < p.rows ? r0 + kColsumRows : p.rows;
+  float acc[8];
+  zero8(acc);
+  for (int64_t r = r0; r < r1; ++r) {
+    float v[8];
+    load8(p.x, p.xbf, r * p.C + col, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += v[e];
+  }
+  store8(p.partial, 0, static_cast<int64_t>(blockIdx.x) * p.C + col, acc);
+}
+
 // ---- host side ----------------------------------------------------------------------------------------------------
 
 inline bool dtype_ok(int d) { return d == DMF_ATTN_F32 || d == DMF_ATTN_BF16; }
@@ -607,6 +637,7 @@ int64_t dmf_block_workspace_floats(int which, int B, int L, int dim) {
     case 0: return static_cast<int64_t>(B) * nchunks(L) * 2 * dim;
     case 1: return static_cast<int64_t>(B) * nchunks(L) * dim;
     case 2: return static_cast<int64_t>(kRmsBlocksMax) * dim;
+    case 3: return ((static_cast<int64_t>(B) * L + kColsumRows - 1) / kColsumRows) * dim;
     default: return 0;
   }
 }
@@ -731,6 +762,23 @@ int dmf_gelu_tanh_fwd(const void* x, const void* tx, void* y, void* ty, int64_t 
 
 int dmf_gelu_tanh_bwd(const void* gy, const void* x, void* gx, int64_t n, int dtype, void* stream) {
   return gelu_impl(x, gy, nullptr, gx, n, dtype, 2, stream);
+}
+
+int dmf_colsum(const void* x, void* out, float* workspace, int64_t rows, int C, int x_dtype, int out_dtype,
+               void* stream) {
+  if (!dtype_ok(x_dtype) || !dtype_ok(out_dtype)) return DMF_ATTN_EDTYPE;
+  if (rows < 1 || C < 8 || C % 8) return DMF_ATTN_ESHAPE;
+  const int64_t nchunk = (rows + kColsumRows - 1) / kColsumRows;
+  if (nchunk > 0x7fffffffLL || C > 8 * kThreads * 65535) return DMF_ATTN_ESHAPE;
+  if (!x || !out || !workspace) return DMF_ATTN_ENULL;
+  if (!aligned16(x) || !aligned16(out) || !aligned16(workspace)) return DMF_ATTN_EALIGN;
+  ColsumParams p{};
+  p.x = x; p.partial = workspace; p.rows = rows; p.C = C; p.xbf = x_dtype == DMF_ATTN_BF16;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(nchunk), static_cast<unsigned>((C / 8 + kThreads - 1) / kThreads));
+  hipLaunchKernelGGL(colsum_kernel, grid, dim3(kThreads), 0, s, p);
+  if (int rc = launch_status()) return rc;
+  return reduce_partials(workspace, out, nullptr, 1, static_cast<int>(nchunk), 1, C, out_dtype == DMF_ATTN_BF16, s);
 }
 
 // Validates a strided (B, L, H, D) operand and copies {sB, sL, sH}.

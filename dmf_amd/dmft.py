@@ -6,7 +6,9 @@ encoder blocks conditioned on (t, y), the remaining decoder blocks and the final
 layer conditioned on (r, y), optional log-variance head.  It exists so that the
 attention kernels can be exercised and timed exactly as the MeanFlow loss calls
 them (``torch.func.jvp`` through the whole model); ``attn_func`` selects the
-operator, ``"hip"`` being this package's kernels.
+operator, ``"hip"`` being this package's kernels, and ``block_ops="hip"`` swaps
+the norm / modulate / gate / GELU glue of every block for the fused kernels of
+``dmf_amd.block_ops``.
 """
 from __future__ import annotations
 
@@ -53,7 +55,8 @@ class DMFT(nn.Module):
         self.pos_embed = nn.Parameter(torch.zeros(1, self.num_patches, hidden_size), requires_grad=False)
         self.blocks = nn.ModuleList(
             [DiTBlock(hidden_size, num_heads, mlp_ratio=mlp_ratio, **block_kwargs) for _ in range(depth)])
-        self.final_layer = FinalLayer(hidden_size, patch_size, self.out_channels)
+        self.final_layer = FinalLayer(hidden_size, patch_size, self.out_channels,
+                                      block_ops=block_kwargs.get("block_ops", "torch"))
         if use_logvar:
             self.logvar_t_embedder = partial(timestep_embedding, dim=128)
             self.logvar_linear = nn.Linear(256, 1)

@@ -51,11 +51,46 @@ def train_step(model, batch, autocast: bool = True):
     return loss
 
 
-def build_model(name: str, attn_func: str, device, qk_norm: bool = False, input_size: int = 32, dmf_depth=None, seed: int = 0):
-    kw = {"attn_func": attn_func, "qk_norm": qk_norm, "input_size": input_size}
+def build_model(name: str, attn_func: str, device, qk_norm: bool = False, input_size: int = 32, dmf_depth=None, seed: int = 0,
+                block_ops: str = "torch"):
+    kw = {"attn_func": attn_func, "qk_norm": qk_norm, "input_size": input_size, "block_ops": block_ops}
     if dmf_depth is not None:
         kw["dmf_depth"] = dmf_depth
     return DMFT_models[name](**kw).init_trunc_normal_(0.02, seed).to(device)
+
+
+class GraphedStep:
+    """A step function captured once into a HIP graph and replayed.
+
+    The uncompiled JVP pass issues roughly a thousand small launches per step
+    from Python (loss.py:165 runs the eager module), which leaves the GPU idle
+    more than half of the time once the kernels themselves are fused; replaying
+    a captured graph removes the host from the loop.  ``fn(*inputs)`` must be a
+    pure function of its tensor arguments (and of module parameters, which are
+    read in place at replay time); its outputs live in the graph's memory pool
+    and are overwritten by the next call.  Capture happens on a side stream at
+    the default priority after ``warmup`` eager calls.
+    """
+
+    def __init__(self, fn, *example_inputs, warmup: int = 3):
+        self.static_inputs = [x.clone() if isinstance(x, torch.Tensor) else x for x in example_inputs]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warmup):
+                fn(*self.static_inputs)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.static_outputs = fn(*self.static_inputs)
+
+    def __call__(self, *inputs):
+        for dst, src in zip(self.static_inputs, inputs):
+            if isinstance(dst, torch.Tensor) and dst is not src:
+                dst.copy_(src)
+        self.graph.replay()
+        return self.static_outputs
 
 
 def _time(fn, steps: int, warmup: int = 2) -> float:
@@ -71,15 +106,17 @@ def _time(fn, steps: int, warmup: int = 2) -> float:
 
 def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True) -> dict:
     """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast, and
-    (b) DMFT-XL/2 256px forward+JVP+backward, batch 32 -- each with the 'hip'
-    operator and, for reference, with the naive 'base' operator."""
+    (b) DMFT-XL/2 256px forward+JVP+backward, batch 32 -- each as ``hip_fused``
+    ('hip' attention + fused block glue), ``hip`` ('hip' attention, the reference's
+    tensor expressions around it) and, for reference, ``base`` (naive attention)."""
     out = {}
     cases = [("DMFT-B/2", 64, 8, False), ("DMFT-XL/2", 32, 20, True)]
+    variants = [("hip_fused", "hip", "hip"), ("hip", "hip", "torch")] + ([("base", "base", "torch")] if compare_base else [])
     for name, batch, dmf_depth, train in cases:
         row = {"batch": batch, "mode": "fwd+jvp+bwd" if train else "fwd+jvp", "dtype": "bf16 autocast"}
         data = synthetic_batch(batch, device)
-        for op in (("hip", "base") if compare_base else ("hip",)):
-            model = build_model(name, op, device, dmf_depth=dmf_depth)
+        for label, op, block_ops in variants:
+            model = build_model(name, op, device, dmf_depth=dmf_depth, block_ops=block_ops)
             if train:
                 def fn():
                     model.zero_grad(set_to_none=True)
@@ -91,8 +128,8 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True) -> di
                     with torch.autocast("cuda", dtype=torch.bfloat16):
                         meanflow_jvp(model, *data)
             sec = _time(fn, steps if op == "hip" else max(2, steps // 2))
-            row[f"{op}_ms_per_step"] = sec * 1e3
-            row[f"{op}_images_per_s"] = batch / sec
+            row[f"{label}_ms_per_step"] = sec * 1e3
+            row[f"{label}_images_per_s"] = batch / sec
             del model
             torch.cuda.empty_cache()
         out[name] = row

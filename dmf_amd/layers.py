@@ -15,10 +15,21 @@ import torch
 import torch.nn as nn
 from torch import Tensor
 
+from . import block_ops as fused
 from .flash_attention_hip_jvp import flash_attn_func as hip_func
 
 # values accepted by --attn-func; "hip" is the one this package adds
 ATTN_FUNCS = ("base", "torch_sdpa", "hip")
+# how the elementwise / normalisation glue of a block runs: "torch" = the reference's
+# tensor expressions (one ATen kernel per primal and per tangent op), "hip" = the fused
+# single-pass kernels of dmf_amd.block_ops
+BLOCK_OPS = ("torch", "hip")
+
+
+def _check_block_ops(block_ops: str) -> bool:
+    if block_ops not in BLOCK_OPS:
+        raise ValueError(f"unknown block_ops {block_ops!r}; expected one of {BLOCK_OPS}")
+    return block_ops == "hip"
 
 
 def attn_op(q: Tensor, k: Tensor, v: Tensor, op: str = "base") -> Tensor:
@@ -45,6 +56,21 @@ def attn_op(q: Tensor, k: Tensor, v: Tensor, op: str = "base") -> Tensor:
     return x.transpose(1, 2)
 
 
+class Linear(nn.Linear):
+    """``nn.Linear`` whose forward-mode pass costs one extra GEMM instead of two
+    (``block_ops.dual_linear``) when ``block_ops="hip"``; parameters, state-dict
+    keys and results are those of ``nn.Linear``."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, block_ops: str = "torch"):
+        super().__init__(in_features, out_features, bias=bias)
+        self.fused = _check_block_ops(block_ops)
+
+    def forward(self, x: Tensor) -> Tensor:
+        if self.fused:
+            return fused.dual_linear(x, self.weight, self.bias)
+        return super().forward(x)
+
+
 def modulate(x: Tensor, shift: Tensor, scale: Tensor) -> Tensor:
     """adaLN modulation (reference models/layers.py:28-29)."""
     return x * (1 + scale) + shift
@@ -53,12 +79,15 @@ def modulate(x: Tensor, shift: Tensor, scale: Tensor) -> Tensor:
 class RMSNorm(nn.Module):
     """Per-head RMS norm over the last dim (reference models/layers.py:33-42)."""
 
-    def __init__(self, dim: int, eps: float = 1e-6):
+    def __init__(self, dim: int, eps: float = 1e-6, block_ops: str = "torch"):
         super().__init__()
         self.eps = eps
         self.scale = nn.Parameter(torch.ones(dim))
+        self.fused = _check_block_ops(block_ops)
 
     def forward(self, x: Tensor) -> Tensor:
+        if self.fused:
+            return fused.rms_norm(x, self.scale, self.eps)
         norm_x = torch.rsqrt(x.pow(2).mean(-1, keepdim=True, dtype=torch.float32) + self.eps)
         return x * norm_x.to(dtype=x.dtype) * self.scale.to(dtype=x.dtype)
 
@@ -66,7 +95,8 @@ class RMSNorm(nn.Module):
 def timestep_embedding(t: Tensor, dim: int, max_period: int = 10000) -> Tensor:
     """Sinusoidal embedding (reference models/layers.py:46-55)."""
     half = dim // 2
-    freqs = torch.exp(-math.log(max_period) * torch.arange(0, half, dtype=torch.float32) / half).to(t.device)
+    # built on t's device (the reference builds it on the host and copies, which a stream capture cannot record)
+    freqs = torch.exp(-math.log(max_period) * torch.arange(0, half, dtype=torch.float32, device=t.device) / half)
     args = t[..., None].float() * freqs[None]
     emb = torch.cat([torch.cos(args), torch.sin(args)], dim=-1)
     if dim % 2:
@@ -104,15 +134,15 @@ class Attention(nn.Module):
     them without a copy."""
 
     def __init__(self, dim: int, num_heads: int = 8, qkv_bias: bool = False, qk_norm: bool = False,
-                 proj_bias: bool = True, attn_func: str = "torch_sdpa") -> None:
+                 proj_bias: bool = True, attn_func: str = "torch_sdpa", block_ops: str = "torch") -> None:
         super().__init__()
         assert dim % num_heads == 0, "dim should be divisible by num_heads"
         self.num_heads = num_heads
         self.head_dim = dim // num_heads
-        self.qkv = nn.Linear(dim, dim * 3, bias=qkv_bias)
-        self.q_norm = RMSNorm(self.head_dim) if qk_norm else nn.Identity()
-        self.k_norm = RMSNorm(self.head_dim) if qk_norm else nn.Identity()
-        self.proj = nn.Linear(dim, dim, bias=proj_bias)
+        self.qkv = Linear(dim, dim * 3, bias=qkv_bias, block_ops=block_ops)
+        self.q_norm = RMSNorm(self.head_dim, block_ops=block_ops) if qk_norm else nn.Identity()
+        self.k_norm = RMSNorm(self.head_dim, block_ops=block_ops) if qk_norm else nn.Identity()
+        self.proj = Linear(dim, dim, bias=proj_bias, block_ops=block_ops)
         self.attn = partial(attn_op, op=attn_func)
 
     def forward(self, x: Tensor) -> Tensor:
@@ -127,11 +157,11 @@ class Attention(nn.Module):
 class Mlp(nn.Module):
     """Reference models/layers.py:158-166."""
 
-    def __init__(self, in_features: int, hidden_features: int):
+    def __init__(self, in_features: int, hidden_features: int, block_ops: str = "torch"):
         super().__init__()
-        self.fc1 = nn.Linear(in_features, hidden_features)
-        self.act = nn.GELU(approximate="tanh")
-        self.fc2 = nn.Linear(hidden_features, in_features)
+        self.fc1 = Linear(in_features, hidden_features, block_ops=block_ops)
+        self.act = fused.gelu_tanh if _check_block_ops(block_ops) else nn.GELU(approximate="tanh")
+        self.fc2 = Linear(hidden_features, in_features, block_ops=block_ops)
 
     def forward(self, x: Tensor) -> Tensor:
         return self.fc2(self.act(self.fc1(x)))
@@ -142,16 +172,21 @@ class DiTBlock(nn.Module):
 
     def __init__(self, hidden_size: int, num_heads: int, mlp_ratio: float = 4.0, **block_kwargs):
         super().__init__()
+        block_ops = block_kwargs.get("block_ops", "torch")
+        self.fused = _check_block_ops(block_ops)
         self.norm1 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
         self.attn = Attention(hidden_size, num_heads=num_heads, qkv_bias=True,
                               qk_norm=block_kwargs.get("qk_norm", False),
-                              attn_func=block_kwargs.get("attn_func", "base"))
+                              attn_func=block_kwargs.get("attn_func", "base"), block_ops=block_ops)
         self.norm2 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
-        self.mlp = Mlp(hidden_size, int(hidden_size * mlp_ratio))
-        self.adaLN_modulation = nn.Sequential(nn.SiLU(), nn.Linear(hidden_size, 6 * hidden_size))
+        self.mlp = Mlp(hidden_size, int(hidden_size * mlp_ratio), block_ops=block_ops)
+        self.adaLN_modulation = nn.Sequential(nn.SiLU(), Linear(hidden_size, 6 * hidden_size, block_ops=block_ops))
 
     def forward(self, x: Tensor, c: Tensor) -> Tensor:
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.adaLN_modulation(c).chunk(6, dim=-1)
+        if self.fused:   # same expressions, each norm+modulate and each gated residual in one kernel
+            x = fused.gate_residual(x, gate_msa, self.attn(fused.ln_modulate(x, shift_msa, scale_msa, self.norm1.eps)))
+            return fused.gate_residual(x, gate_mlp, self.mlp(fused.ln_modulate(x, shift_mlp, scale_mlp, self.norm2.eps)))
         x = x + gate_msa * self.attn(modulate(self.norm1(x), shift_msa, scale_msa))
         x = x + gate_mlp * self.mlp(modulate(self.norm2(x), shift_mlp, scale_mlp))
         return x
@@ -160,14 +195,17 @@ class DiTBlock(nn.Module):
 class FinalLayer(nn.Module):
     """Reference models/layers.py:205-220."""
 
-    def __init__(self, hidden_size: int, patch_size: int, out_channels: int):
+    def __init__(self, hidden_size: int, patch_size: int, out_channels: int, block_ops: str = "torch"):
         super().__init__()
+        self.fused = _check_block_ops(block_ops)
         self.norm_final = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
-        self.linear = nn.Linear(hidden_size, patch_size * patch_size * out_channels)
-        self.adaLN_modulation = nn.Sequential(nn.SiLU(), nn.Linear(hidden_size, 2 * hidden_size))
+        self.linear = Linear(hidden_size, patch_size * patch_size * out_channels, block_ops=block_ops)
+        self.adaLN_modulation = nn.Sequential(nn.SiLU(), Linear(hidden_size, 2 * hidden_size, block_ops=block_ops))
 
     def forward(self, x: Tensor, c: Tensor) -> Tensor:
         shift, scale = self.adaLN_modulation(c).chunk(2, dim=-1)
+        if self.fused:
+            return self.linear(fused.ln_modulate(x, shift, scale, self.norm_final.eps))
         return self.linear(modulate(self.norm_final(x), shift, scale))
 
 

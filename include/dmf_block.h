@@ -40,7 +40,8 @@ extern "C" {
 
 /* Number of fp32 workspace elements a backward entry point needs.
  * `which`: 0 = dmf_ln_modulate_bwd, 1 = dmf_gate_residual_bwd (rows = B*L, dim = C),
- *          2 = dmf_rmsnorm_bwd (rows = B*L*H, dim = D).  Returns 0 on bad input. */
+ *          2 = dmf_rmsnorm_bwd (dim = D; B, L ignored), 3 = dmf_colsum (rows = B*L, dim = C).
+ * Returns 0 on bad input. */
 DMF_ATTN_API int64_t dmf_block_workspace_floats(int which, int B, int L, int dim);
 
 /*
@@ -124,6 +125,15 @@ DMF_ATTN_API int dmf_rmsnorm_fwd(const void* x, const void* tx, const void* gain
 DMF_ATTN_API int dmf_rmsnorm_bwd(const void* gy, const void* x, const void* gain, void* gx, void* ggain,
                                  float* workspace, const int64_t* strides, int B, int L, int H, int D, float eps,
                                  int dtype, int gain_dtype, void* stream);
+
+/*
+ * out[c] = sum_r x[r][c] for a dense (rows, C) matrix, C a multiple of 8: the
+ * bias gradient of a Linear layer (the `grad_output.sum(0)` of torch's
+ * `linear_backward`, reached from models/layers.py:131,137,161-165) as a
+ * fixed-order two-stage sum, safe to record into a HIP graph.
+ */
+DMF_ATTN_API int dmf_colsum(const void* x, void* out, float* workspace, int64_t rows, int C, int x_dtype,
+                            int out_dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -179,3 +179,29 @@ def test_block_abi_rejects_bad_arguments():
         _lib.gate_residual_fwd(big, torch.zeros(1, 4096, device=DEV), big)
     with pytest.raises(RuntimeError, match="head dim"):
         _lib.rmsnorm_fwd(torch.zeros(1, 2, 2, 20, device=DEV), torch.ones(20, device=DEV))
+
+
+@pytest.mark.parametrize("rows,C", [(1000, 2304), (1, 8), (16384, 768), (77, 4608)])
+@pytest.mark.parametrize("dt", [F32, BF16])
+def test_colsum(rows, C, dt):
+    print(f"colsum {rows}x{C} {dt}", flush=True)
+    x = torch.randn(rows, C, generator=torch.Generator().manual_seed(17)).to(dt)
+    got = _lib.colsum(x.to(DEV), torch.float32)
+    _close(got, x.double().sum(0), 1e-5, "colsum")
+    assert torch.equal(got, _lib.colsum(x.to(DEV), torch.float32))   # fixed summation order
+
+
+def test_dual_linear_under_func_jvp_and_autograd():
+    from torch.nn.functional import linear
+    g = torch.Generator().manual_seed(18)
+    x, tx, gy = torch.randn(2, 24, 64, generator=g), torch.randn(2, 24, 64, generator=g), torch.randn(2, 24, 48, generator=g)
+    w, b = torch.randn(48, 64, generator=g) * 0.1, torch.randn(48, generator=g)
+    xd, wd, bd = x.to(DEV).requires_grad_(), w.to(DEV).requires_grad_(), b.to(DEV).requires_grad_()
+    y, ty = torch.func.jvp(lambda a: block_ops.dual_linear(a, wd, bd), (xd,), (tx.to(DEV),))
+    _close(y, linear(x, w, b), 1e-5, "y")
+    _close(ty, linear(tx, w), 1e-5, "ty")
+    (y * gy.to(DEV)).sum().backward()
+    gx, gw, gb = bo.grads(lambda a, ww, bb: linear(a, ww, bb), (x, w, b), gy)
+    _close(xd.grad, gx, 1e-5, "gx")
+    _close(wd.grad, gw, 1e-5, "gw")
+    _close(bd.grad, gb, 1e-5, "gb")

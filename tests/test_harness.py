@@ -89,3 +89,57 @@ def test_dmft_hip_qk_norm_no_grad_sampling_path():
     z, t, r, y, _ = harness.synthetic_batch(2, dev)
     with torch.no_grad():
         assert ao.rel_l2(m_hip(z, t, r, y).cpu(), m_base(z, t, r, y).cpu()) < 1e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("autocast,tol", [(False, 2e-4), (True, 3e-2)])
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_dmft_fused_block_ops_vs_torch_block_ops(autocast, tol, qk_norm):
+    """Same model, weights and inputs; block glue (norm+modulate, gated residual,
+    GELU, qk RMSNorm) through the fused kernels vs the reference's tensor
+    expressions, both around the naive 'base' attention and around the 'hip' one.
+    Under autocast the reference expressions round intermediate products to bf16
+    (models/layers.py:29,42,198) where the fused kernels round once, hence the
+    bf16-level tolerance there."""
+    dev = "cuda:0"
+    kw = dict(input_size=32, hidden_size=288, depth=4, num_heads=4, dmf_depth=3, qk_norm=qk_norm)
+    m_ref = _small("base", **kw).to(dev)
+    with torch.no_grad():   # non-trivial RMSNorm gains
+        for n, p in m_ref.named_parameters():
+            if n.endswith("_norm.scale"):
+                p.copy_(1 + 0.1 * torch.randn(p.shape, generator=torch.Generator().manual_seed(7)).to(dev))
+    data = harness.synthetic_batch(4, dev)
+
+    def run(m):
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            loss, u, du = harness.meanflow_loss(m, *data)
+        loss.backward()
+        return u.float().cpu(), du.float().cpu()
+
+    u_ref, du_ref = run(m_ref)
+    for attn in ("base", "hip"):
+        m = _small(attn, block_ops="hip", **kw).to(dev)
+        m.load_state_dict(m_ref.state_dict())
+        u, du = run(m)
+        assert ao.rel_l2(u, u_ref) <= tol, (attn, ao.rel_l2(u, u_ref))
+        assert ao.rel_l2(du, du_ref) <= tol, (attn, ao.rel_l2(du, du_ref))
+        worst = max((ao.rel_l2(p.grad.cpu(), q.grad.cpu()), n) for (n, p), (_, q) in zip(m.named_parameters(), m_ref.named_parameters())
+                    if q.grad is not None and float(q.grad.abs().max()) > 0)
+        assert all(p.grad is not None for (n, p), (_, q) in zip(m.named_parameters(), m_ref.named_parameters()) if q.grad is not None)
+        assert worst[0] <= 5 * tol, (attn, worst)
+
+
+@pytest.mark.gpu
+def test_dmft_fused_block_ops_no_grad_and_plain_forward():
+    dev = "cuda:0"
+    kw = dict(input_size=32, hidden_size=288, depth=2, num_heads=4, dmf_depth=1, qk_norm=True)
+    m_f, m_ref = _small("hip", block_ops="hip", **kw).to(dev), _small("base", **kw).to(dev)
+    m_ref.load_state_dict(m_f.state_dict())
+    z, t, r, y, _ = harness.synthetic_batch(2, dev)
+    with torch.no_grad():
+        assert ao.rel_l2(m_f(z, t, r, y).cpu(), m_ref(z, t, r, y).cpu()) < 1e-4
+
+
+def test_unknown_block_ops_raises():
+    with pytest.raises(ValueError):
+        _small("base", block_ops="nope")

@@ -1,5 +1,5 @@
 """CPU-only tests: the C-ABI library loads and exports what include/dmf_attn.h
-declares, argument validation returns the documented codes (no kernel is
+and include/dmf_block.h declare, argument validation returns the documented codes (no kernel is
 launched on those paths), and the autograd / forward-AD protocol of the Python
 operator behaves like the reference's (models/flash_attention_2_jvp.py:177-319)
 when the three kernel calls are replaced by stand-ins defined in this file."""
@@ -19,14 +19,17 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "dmf_attn.h")).read()
-    return re.findall(r"DMF_ATTN_API\s+[\w\s\*]+?\b(dmf_attn_\w+)\s*\(", text)
+    names = []
+    for header in ("dmf_attn.h", "dmf_block.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        names += re.findall(r"DMF_ATTN_API\s+[\w\s\*]+?\b(dmf_\w+)\s*\(", text)
+    return names
 
 
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = _declared_symbols()
-    assert set(names) == set(_lib.SIGNATURES), names
+    assert len(names) == 15 and set(names) == set(_lib.SIGNATURES), names
     for n in names:
         assert getattr(lib, n) is not None
     assert lib.dmf_attn_version() >= 1
@@ -184,3 +187,31 @@ def test_rmsnorm_and_pos_embed_match_oracle_formulas():
     assert abs(pe[0, :4]).max() == 0 and (pe[0, 4:8] == 1).all()
     assert pe[1, 0] == pytest.approx(float(torch.sin(torch.tensor(1.0))))   # token 1 = (row 0, col 1)
     assert pe[4, 8] == pytest.approx(float(torch.sin(torch.tensor(1.0))))   # token 4 = (row 1, col 0)
+
+
+def test_block_abi_validation_codes_without_launch():
+    """Argument checks of the block-glue entry points return before any launch."""
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(1 << 16)
+    p = (ctypes.addressof(buf) + 15) // 16 * 16
+    ms = (ctypes.c_int64 * 4)(64, 64, 64, 64)
+    ln = lambda **kw: lib.dmf_ln_modulate_fwd(
+        kw.get("x", p), None, p, kw.get("scale", p), None, None, p, None, kw.get("ms", ms), kw.get("B", 2), 4, kw.get("C", 64),
+        1e-6, kw.get("dt", 0), 0, 0, None)
+    assert ln(C=20) == -3 and ln(C=4096) == -3 and ln(B=0) == -3
+    assert ln(dt=5) == -1
+    assert ln(x=None) == -5 and ln(scale=None) == -5
+    assert ln(x=p + 8) == -6
+    assert ln(ms=(ctypes.c_int64 * 4)(64, 66, 64, 64)) == -4
+    assert lib.dmf_gelu_tanh_fwd(p, None, p, None, 12, 0, None) == -3      # n not a multiple of 8
+    assert lib.dmf_gelu_tanh_fwd(p, None, p, p, 16, 0, None) == -5         # tangent output without tangent input
+    assert lib.dmf_gelu_tanh_bwd(None, p, p, 16, 0, None) == -5
+    st = (ctypes.c_int64 * 8)(*([4 * 2 * 24, 2 * 24, 24, 1] * 2))
+    assert lib.dmf_rmsnorm_fwd(p, None, p, p, None, st, 1, 4, 2, 20, 1e-6, 0, 0, None) == -2   # head dim
+    bad = (ctypes.c_int64 * 8)(*([4 * 2 * 24, 2 * 24, 24, 2] * 2))
+    assert lib.dmf_rmsnorm_fwd(p, None, p, p, None, bad, 1, 4, 2, 24, 1e-6, 0, 0, None) == -4
+    assert lib.dmf_gate_residual_bwd(p, p, p, p, p, None, 64, 2, 4, 64, 0, 0, 0, None) == -5   # workspace missing
+    assert lib.dmf_block_workspace_floats(0, 2, 33, 64) == 2 * 2 * 2 * 64
+    assert lib.dmf_block_workspace_floats(1, 2, 33, 64) == 2 * 2 * 64
+    assert lib.dmf_block_workspace_floats(2, 1, 1, 72) == 1024 * 72
+    assert lib.dmf_block_workspace_floats(9, 1, 1, 72) == 0
