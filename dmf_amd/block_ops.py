@@ -131,35 +131,48 @@ class RMSNormFunc(torch.autograd.Function):
 
 
 class DualLinearFunc(torch.autograd.Function):
-    """(x, tx, weight, bias) -> (y, ty) = (x W^T + b, tx W^T): exactly one library
-    GEMM per stream.  torch's own forward-mode rule for ``linear`` also multiplies
-    the primal input by a materialised all-zero weight tangent and adds the two
-    products (three GEMMs, two fills, a copy and an add per layer); parameters
-    carry no tangent in the MeanFlow JVP (loss.py:165-170), so that work is
-    skipped here.  Runs under autocast like ``F.linear``."""
+    """(x, tx, weight, bias) -> (y, ty, w) with y = x W^T + b, ty = tx W^T: exactly
+    one library GEMM per stream.  torch's own forward-mode rule for ``linear``
+    also multiplies the primal input by a materialised all-zero weight tangent
+    and adds the two products (three GEMMs, two fills, a copy and an add per
+    layer); parameters carry no tangent in the MeanFlow JVP (loss.py:165-170), so
+    that work is skipped here.  Under autocast the operands are cast once (``w``,
+    the cast weight, is returned so that ``backward`` can reuse it)."""
 
     @staticmethod
     def forward(x, tx, weight, bias):
-        y = torch.nn.functional.linear(x, weight, bias)
-        ty = None if tx is None else torch.nn.functional.linear(tx, weight)
-        return y, ty
+        linear = torch.nn.functional.linear
+        if x.is_cuda and torch.is_autocast_enabled("cuda"):
+            dt = torch.get_autocast_dtype("cuda")
+            w = weight.to(dt)
+            b = None if bias is None else bias.to(dt)
+            with torch.autocast("cuda", enabled=False):
+                y = linear(x.to(dt), w, b)
+                ty = None if tx is None else linear(tx.to(dt), w)
+            return y, ty, (w if w is not weight else None)
+        return linear(x, weight, bias), (None if tx is None else linear(tx, weight)), None
 
     @staticmethod
     def setup_context(ctx, inputs, outputs):
         x, _, weight, bias = inputs
-        ctx.save_for_backward(x, weight)
+        w = outputs[2]
+        ctx.save_for_backward(x, weight if w is None else w)
+        ctx.weight_dtype = weight.dtype
         ctx.bias_dtype = None if bias is None else bias.dtype
+        if w is not None:
+            ctx.mark_non_differentiable(w)
         ctx.set_materialize_grads(False)
 
     @staticmethod
-    def backward(ctx, gy, gty):
+    def backward(ctx, gy, gty, gw_unused):
         if gy is None:
             return None, None, None, None
-        x, weight = ctx.saved_tensors
-        g2 = gy.reshape(-1, gy.shape[-1])
-        x2 = x.reshape(-1, x.shape[-1]).to(g2.dtype)
-        gx = (g2 @ weight.to(g2.dtype)).reshape(x.shape).to(x.dtype) if ctx.needs_input_grad[0] else None
-        gw = (g2.t() @ x2).to(weight.dtype) if ctx.needs_input_grad[2] else None
+        x, w = ctx.saved_tensors
+        g2 = gy.reshape(-1, gy.shape[-1]).to(w.dtype)
+        gx = (g2 @ w).reshape(x.shape).to(x.dtype) if ctx.needs_input_grad[0] else None
+        gw = None
+        if ctx.needs_input_grad[2]:
+            gw = (g2.t() @ x.reshape(-1, x.shape[-1]).to(w.dtype)).to(ctx.weight_dtype)
         gb = None
         if ctx.bias_dtype is not None and ctx.needs_input_grad[3]:
             # torch's multi-block column reduction clears its scratch with a memset node, which does not survive
@@ -172,7 +185,7 @@ def dual_linear(x, weight, bias=None):
     """``F.linear(x, weight, bias)``; a forward-AD dual ``x`` gives a dual result
     (weight and bias are constants of the tangent map)."""
     (xp,), (tx,), dual = _unpack(x)
-    y, ty = DualLinearFunc.apply(xp, tx, weight, bias)
+    y, ty, _ = DualLinearFunc.apply(xp, tx, weight, bias)
     return fwAD.make_dual(y, ty) if dual else y
 
 

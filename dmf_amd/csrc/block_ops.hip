@@ -545,9 +545,10 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(RmsParams p) {
 }
 
 // ---- column sums of a dense (rows, C) matrix ----------------------------------------------------------------------
-// Work-group (x, y): rows [x*kColsumRows, +kColsumRows), vector columns y*kThreads + thread.
+// Work-group (x, y): rows [x*kColsumRows, +kColsumRows), 64 vector columns starting at y*64.  Wave w takes rows
+// w, w+4, ... of the chunk (four loads in flight per lane), the four waves are added through LDS.
 
-constexpr int kColsumRows = 64;
+constexpr int kColsumRows = 256;
 
 struct ColsumParams {
   const void* x;
@@ -558,19 +559,41 @@ struct ColsumParams {
 };
 
 __global__ __launch_bounds__(kThreads) void colsum_kernel(ColsumParams p) {
-  const int col = (blockIdx.y * kThreads + threadIdx.x) * 8;
-  if (col >= p.C) return;
+  __shared__ float lds[kWaves - 1][64 * 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = (blockIdx.y * 64 + lane) * 8;
+  const bool live = col < p.C;
   const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kColsumRows;
   const int64_t r1 = r0 + kColsumRows < p.rows ? r0 + kColsumRows : p.rows;
   float acc[8];
   zero8(acc);
-  for (int64_t r = r0; r < r1; ++r) {
-    float v[8];
-    load8(p.x, p.xbf, r * p.C + col, v);
+  if (live) {
+    int64_t r = r0 + wave;
+    for (; r + 3 * kWaves < r1; r += 4 * kWaves) {
+      float v[4][8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += v[e];
+      for (int u = 0; u < 4; ++u) load8(p.x, p.xbf, (r + u * kWaves) * p.C + col, v[u]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (v[0][e] + v[1][e]) + (v[2][e] + v[3][e]);
+    }
+    for (; r < r1; r += kWaves) {
+      float v[8];
+      load8(p.x, p.xbf, r * p.C + col, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += v[e];
+    }
   }
-  store8(p.partial, 0, static_cast<int64_t>(blockIdx.x) * p.C + col, acc);
+  if (wave > 0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) lds[wave - 1][lane * 8 + e] = acc[e];
+  }
+  __syncthreads();
+  if (wave == 0 && live) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      for (int w = 0; w < kWaves - 1; ++w) acc[e] += lds[w][lane * 8 + e];
+    store8(p.partial, 0, static_cast<int64_t>(blockIdx.x) * p.C + col, acc);
+  }
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------
@@ -769,13 +792,13 @@ int dmf_colsum(const void* x, void* out, float* workspace, int64_t rows, int C, 
   if (!dtype_ok(x_dtype) || !dtype_ok(out_dtype)) return DMF_ATTN_EDTYPE;
   if (rows < 1 || C < 8 || C % 8) return DMF_ATTN_ESHAPE;
   const int64_t nchunk = (rows + kColsumRows - 1) / kColsumRows;
-  if (nchunk > 0x7fffffffLL || C > 8 * kThreads * 65535) return DMF_ATTN_ESHAPE;
+  if (nchunk > 0x7fffffffLL || C > 8 * 64 * 65535) return DMF_ATTN_ESHAPE;
   if (!x || !out || !workspace) return DMF_ATTN_ENULL;
   if (!aligned16(x) || !aligned16(out) || !aligned16(workspace)) return DMF_ATTN_EALIGN;
   ColsumParams p{};
   p.x = x; p.partial = workspace; p.rows = rows; p.C = C; p.xbf = x_dtype == DMF_ATTN_BF16;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(nchunk), static_cast<unsigned>((C / 8 + kThreads - 1) / kThreads));
+  const dim3 grid(static_cast<unsigned>(nchunk), static_cast<unsigned>((C / 8 + 63) / 64));
   hipLaunchKernelGGL(colsum_kernel, grid, dim3(kThreads), 0, s, p);
   if (int rc = launch_status()) return rc;
   return reduce_partials(workspace, out, nullptr, 1, static_cast<int>(nchunk), 1, C, out_dtype == DMF_ATTN_BF16, s);

@@ -18,7 +18,9 @@ import torch
 import torch.nn as nn
 from torch import Tensor
 
-from .layers import DiTBlock, FinalLayer, LabelEmbedder, TimestepEmbedder, get_2d_sincos_pos_embed, timestep_embedding
+from . import block_ops as block_ops_mod
+from .layers import (DiTBlock, FinalLayer, LabelEmbedder, TimestepEmbedder, _check_block_ops, get_2d_sincos_pos_embed,
+                     timestep_embedding)
 
 
 class PatchEmbed(nn.Module):
@@ -26,14 +28,23 @@ class PatchEmbed(nn.Module):
     output as the ``timm`` layer the reference uses (models/dmft.py:15,54-56):
     ``proj = Conv2d(C_in, C, kernel=stride=patch)``, tokens in row-major order."""
 
-    def __init__(self, img_size: int, patch_size: int, in_chans: int, embed_dim: int, bias: bool = True):
+    def __init__(self, img_size: int, patch_size: int, in_chans: int, embed_dim: int, bias: bool = True,
+                 block_ops: str = "torch"):
         super().__init__()
         self.patch_size = patch_size
         self.num_patches = (img_size // patch_size) ** 2
         self.proj = nn.Conv2d(in_chans, embed_dim, kernel_size=patch_size, stride=patch_size, bias=bias)
+        self.fused = _check_block_ops(block_ops)
 
     def forward(self, x: Tensor) -> Tensor:
-        return self.proj(x).flatten(2).transpose(1, 2)
+        if not self.fused:
+            return self.proj(x).flatten(2).transpose(1, 2)
+        # kernel == stride, so the convolution is a Linear over flattened (C_in, p, p) patches: one small GEMM
+        # (and GEMM gradients) instead of the generic convolution path
+        B, C, H, W = x.shape
+        p = self.patch_size
+        patches = x.reshape(B, C, H // p, p, W // p, p).permute(0, 2, 4, 1, 3, 5).reshape(B, (H // p) * (W // p), C * p * p)
+        return block_ops_mod.dual_linear(patches, self.proj.weight.reshape(self.proj.out_channels, -1), self.proj.bias)
 
 
 class DMFT(nn.Module):
@@ -48,7 +59,8 @@ class DMFT(nn.Module):
         self.num_heads, self.num_classes = num_heads, num_classes
         self.dmf_depth, self.use_logvar = dmf_depth, use_logvar
 
-        self.x_embedder = PatchEmbed(input_size, patch_size, in_channels, hidden_size, bias=True)
+        self.x_embedder = PatchEmbed(input_size, patch_size, in_channels, hidden_size, bias=True,
+                                     block_ops=block_kwargs.get("block_ops", "torch"))
         self.t_embedder = TimestepEmbedder(hidden_size)
         self.y_embedder = LabelEmbedder(num_classes, hidden_size, use_cfg_embedding)
         self.num_patches = self.x_embedder.num_patches

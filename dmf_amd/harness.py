@@ -106,31 +106,36 @@ def _time(fn, steps: int, warmup: int = 2) -> float:
 
 def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True) -> dict:
     """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast, and
-    (b) DMFT-XL/2 256px forward+JVP+backward, batch 32 -- each as ``hip_fused``
-    ('hip' attention + fused block glue), ``hip`` ('hip' attention, the reference's
-    tensor expressions around it) and, for reference, ``base`` (naive attention)."""
+    (b) DMFT-XL/2 256px forward+JVP+backward, batch 32.  Variants:
+    ``hip_fused_graph`` -- 'hip' attention + fused block glue, replayed as a HIP graph,
+    ``hip_fused``       -- the same, launched eagerly from Python,
+    ``hip``             -- 'hip' attention inside the reference's tensor expressions,
+    ``base``            -- naive attention (the reference's own CPU-runnable operator)."""
     out = {}
     cases = [("DMFT-B/2", 64, 8, False), ("DMFT-XL/2", 32, 20, True)]
-    variants = [("hip_fused", "hip", "hip"), ("hip", "hip", "torch")] + ([("base", "base", "torch")] if compare_base else [])
+    variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused", "hip", "hip", False), ("hip", "hip", "torch", False)]
+    if compare_base:
+        variants.append(("base", "base", "torch", False))
     for name, batch, dmf_depth, train in cases:
         row = {"batch": batch, "mode": "fwd+jvp+bwd" if train else "fwd+jvp", "dtype": "bf16 autocast"}
         data = synthetic_batch(batch, device)
-        for label, op, block_ops in variants:
+        for label, op, block_ops, graphed in variants:
             model = build_model(name, op, device, dmf_depth=dmf_depth, block_ops=block_ops)
             if train:
-                def fn():
+                def step(*batch_tensors):
                     model.zero_grad(set_to_none=True)
-                    train_step(model, data)
+                    return train_step(model, batch_tensors).detach()
             else:
                 model.requires_grad_(False)
 
-                def fn():
+                def step(*batch_tensors):
                     with torch.autocast("cuda", dtype=torch.bfloat16):
-                        meanflow_jvp(model, *data)
-            sec = _time(fn, steps if op == "hip" else max(2, steps // 2))
+                        return meanflow_jvp(model, *batch_tensors)
+            run = GraphedStep(step, *data) if graphed else step
+            sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
             row[f"{label}_ms_per_step"] = sec * 1e3
             row[f"{label}_images_per_s"] = batch / sec
-            del model
+            del model, run, step
             torch.cuda.empty_cache()
         out[name] = row
     return out

@@ -143,3 +143,16 @@ def test_dmft_fused_block_ops_no_grad_and_plain_forward():
 def test_unknown_block_ops_raises():
     with pytest.raises(ValueError):
         _small("base", block_ops="nope")
+
+
+def test_patch_embed_equals_strided_convolution():
+    """models/dmft.py:54-56 uses timm's PatchEmbed (a kernel=stride convolution); the
+    harness evaluates it as a Linear over flattened patches with the same parameters."""
+    from dmf_amd.dmft import PatchEmbed
+    pe = PatchEmbed(16, 4, 3, 40, block_ops="hip").double()
+    x = torch.randn(2, 3, 16, 16, dtype=torch.float64)
+    ref = pe.proj(x).flatten(2).transpose(1, 2)
+    assert torch.allclose(pe(x), ref, atol=1e-12)
+    pe.fused = False
+    assert torch.equal(pe(x), ref)
+    assert pe.proj.weight.shape == (40, 3, 4, 4)
