@@ -12,7 +12,8 @@ bf16, q/k RMS-normalised), inputs resident in HBM.  Prints ONE JSON line:
                  timed on this box's host cores on a bounded slice of the
                  same workload
   extra          the other kernel-level figures (N=256 shape, backward,
-                 primal-only forward) and DMFT forward+JVP images/s
+                 primal-only forward, the HBM-bound block-glue kernels) and
+                 DMFT forward+JVP / train-step images/s
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
 """
@@ -179,6 +180,41 @@ def device_probes():
     return out
 
 
+def block_kernel_rows(device, steps=50, warmup=10):
+    """HBM-bound block-glue kernels at the two end-to-end shapes: algorithmic
+    bytes (each operand read once, each result written once) / launch time."""
+    import torch
+    from dmf_amd import _lib
+
+    out = {}
+    f32, bf16 = torch.float32, torch.bfloat16
+    for tag, (B, L, C) in {"dmft_b2_b64": (64, 256, 768), "dmft_xl2_b32": (32, 256, 1152)}.items():
+        n = B * L * C
+        x, tx, gyf = (torch.randn(B, L, C, device=device) for _ in range(3))
+        h, th, gyb = (torch.randn(B, L, C, device=device, dtype=bf16) for _ in range(3))
+        mods = torch.randn(B, 1, 6 * C, device=device, dtype=bf16) * 0.3
+        tmods = torch.randn(B, 1, 6 * C, device=device, dtype=bf16) * 0.3
+        sh, sc, gt = mods[..., :C], mods[..., C:2 * C], mods[..., 2 * C:3 * C]
+        tsh, tsc, tgt = tmods[..., :C], tmods[..., C:2 * C], tmods[..., 2 * C:3 * C]
+        u, tu = (torch.randn(B, L, 4 * C, device=device, dtype=bf16) for _ in range(2))
+        cases = {
+            # name: (callable, algorithmic bytes)
+            "ln_modulate_fwd_jvp": (lambda: _lib.ln_modulate_fwd(x, sh, sc, tx, tsh, tsc, 1e-6, bf16, True), n * (4 + 4 + 2 + 2)),
+            "ln_modulate_bwd": (lambda: _lib.ln_modulate_bwd(gyb, x, sc), n * (2 + 4 + 4)),
+            "gate_residual_fwd_jvp": (lambda: _lib.gate_residual_fwd(x, gt, h, tx, tgt, th, True), n * (4 + 4 + 2 + 2 + 4 + 4)),
+            "gate_residual_bwd": (lambda: _lib.gate_residual_bwd(gyf, gt, h), n * (4 + 2 + 2)),
+            "gelu_tanh_fwd_jvp": (lambda: _lib.gelu_tanh_fwd(u, tu), 4 * n * 2 * 4),
+            "gelu_tanh_bwd": (lambda: _lib.gelu_tanh_bwd(tu, u), 4 * n * 2 * 3),
+            "colsum_4C": (lambda: _lib.colsum(u.view(B * L, 4 * C), f32), 4 * n * 2),
+        }
+        row = {}
+        for kname, (fn, nbytes) in cases.items():
+            ms, _ = time_gpu(fn, steps, warmup)
+            row[kname] = {"ms": ms, "hbm_gbs_algorithmic": nbytes / ms / 1e6, "pct_hbm_peak": 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS}
+        out[tag] = row
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -250,6 +286,7 @@ def main():
             extra[wname] = row
             del ins
         extra["device_probes"] = device_probes()
+        extra["block_kernels"] = block_kernel_rows(dev)
         try:
             from dmf_amd import harness
             extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10))

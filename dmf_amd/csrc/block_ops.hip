@@ -22,7 +22,7 @@ namespace blk {
 
 constexpr int kWaves = 4;          // waves per work-group
 constexpr int kThreads = 64 * kWaves;
-constexpr int kChunkRows = 32;     // rows of one sample handled by one work-group in the reducing backward kernels
+constexpr int kChunkRows = 16;     // rows of one sample handled by one work-group in the reducing backward kernels
 constexpr int kMaxC = 2048;        // 4 vectors of 8 per lane
 constexpr int kRmsBlocksMax = 1024;
 

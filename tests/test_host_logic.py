@@ -211,7 +211,7 @@ def test_block_abi_validation_codes_without_launch():
     bad = (ctypes.c_int64 * 8)(*([4 * 2 * 24, 2 * 24, 24, 2] * 2))
     assert lib.dmf_rmsnorm_fwd(p, None, p, p, None, bad, 1, 4, 2, 24, 1e-6, 0, 0, None) == -4
     assert lib.dmf_gate_residual_bwd(p, p, p, p, p, None, 64, 2, 4, 64, 0, 0, 0, None) == -5   # workspace missing
-    assert lib.dmf_block_workspace_floats(0, 2, 33, 64) == 2 * 2 * 2 * 64
-    assert lib.dmf_block_workspace_floats(1, 2, 33, 64) == 2 * 2 * 64
+    assert lib.dmf_block_workspace_floats(0, 2, 33, 64) == 2 * 3 * 2 * 64
+    assert lib.dmf_block_workspace_floats(1, 2, 33, 64) == 2 * 3 * 64
     assert lib.dmf_block_workspace_floats(2, 1, 1, 72) == 1024 * 72
     assert lib.dmf_block_workspace_floats(9, 1, 1, 72) == 0
