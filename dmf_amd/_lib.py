@@ -38,6 +38,8 @@ SIGNATURES = {
     "dmf_rmsnorm_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_rmsnorm_bwd": (c_int, [_P] * 6 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_colsum": (c_int, [_P] * 3 + [_L, _I, _I, _I, _P]),
+    "dmf_silu_fwd": (c_int, [_P] * 4 + [_L, _I, _I, _P]),
+    "dmf_silu_bwd": (c_int, [_P] * 3 + [_L, _I, _I, _P]),
 }
 
 _lib = None
@@ -365,3 +367,27 @@ def colsum(x, out_dtype=None):
         rc = load().dmf_colsum(x.data_ptr(), out.data_ptr(), ws.data_ptr(), rows, C, _dtype_code(x), _dtype_code(out), _stream(x))
     _check(rc, "dmf_colsum")
     return out
+
+
+def silu_fwd(x, tx=None, out_dtype=None):
+    """(y, ty) of SiLU in ``out_dtype`` (default: x's); ty is None when ``tx`` is None."""
+    if not x.is_cuda:
+        raise RuntimeError("dmf_amd block kernels run on the GPU only (tensor is on %s)" % x.device)
+    _same_dtype("silu", x, tx)
+    x, tx = _dense(x), _dense(tx)
+    out_dtype = out_dtype or x.dtype
+    y = _empty(x.shape, out_dtype, x.device)
+    ty = _empty(x.shape, out_dtype, x.device) if tx is not None else None
+    with torch.cuda.device(x.device):
+        rc = load().dmf_silu_fwd(x.data_ptr(), _ptr(tx), y.data_ptr(), _ptr(ty), x.numel(), _dtype_code(x), _dtype_code(y), _stream(x))
+    _check(rc, "dmf_silu_fwd")
+    return y, ty
+
+
+def silu_bwd(gy, x):
+    gy, x = _dense(gy), _dense(x)
+    gx = _empty(x.shape, x.dtype, x.device)
+    with torch.cuda.device(x.device):
+        rc = load().dmf_silu_bwd(gy.data_ptr(), x.data_ptr(), gx.data_ptr(), x.numel(), _dtype_code(x), _dtype_code(gy), _stream(x))
+    _check(rc, "dmf_silu_bwd")
+    return gx

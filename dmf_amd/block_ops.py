@@ -7,6 +7,7 @@ attention operator in the reference's block (models/layers.py):
 * ``gate_residual(x, gate, h)``     = ``x + gate * h``                           (:198, :200)
 * ``gelu_tanh(x)``                  = ``nn.GELU(approximate="tanh")(x)``         (:162, :166)
 * ``rms_norm(x, gain)``             = ``RMSNorm.forward``                        (:33-42, :148)
+* ``silu(x)``                       = ``nn.SiLU()`` of the adaLN branch          (:185-188, :211-214)
 * ``dual_linear(x, weight, bias)``  = ``nn.Linear`` (:131,137,161-165,...) -- library GEMMs, see ``DualLinearFunc``
 
 Each follows the protocol of the attention operator (flash_attention_hip_jvp):
@@ -105,6 +106,26 @@ class GeluTanhFunc(torch.autograd.Function):
             return None, None
         (x,) = ctx.saved_tensors
         return _lib.gelu_tanh_bwd(gy.to(x.dtype), x), None
+
+
+class SiluFunc(torch.autograd.Function):
+    """(x, tx, out_dtype) -> (y, ty)."""
+
+    @staticmethod
+    def forward(x, tx, out_dtype):
+        return _lib.silu_fwd(x, tx, out_dtype)
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        ctx.save_for_backward(inputs[0])
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, gy, gty):
+        if gy is None:
+            return None, None, None
+        (x,) = ctx.saved_tensors
+        return _lib.silu_bwd(gy, x), None, None
 
 
 class RMSNormFunc(torch.autograd.Function):
@@ -220,6 +241,14 @@ def gelu_tanh(x):
     """tanh-approximated GELU."""
     (xp,), (tx,), dual = _unpack(x)
     y, ty = GeluTanhFunc.apply(xp, tx)
+    return fwAD.make_dual(y, ty) if dual else y
+
+
+def silu(x):
+    """``x * sigmoid(x)``; under autocast the result is produced in the autocast
+    dtype (it feeds the adaLN projection, which would cast it)."""
+    (xp,), (tx,), dual = _unpack(x)
+    y, ty = SiluFunc.apply(xp, tx, _autocast_dtype(xp))
     return fwAD.make_dual(y, ty) if dual else y
 
 

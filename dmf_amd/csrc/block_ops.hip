@@ -390,40 +390,49 @@ __global__ __launch_bounds__(kThreads) void gate_residual_bwd_kernel(GateBwdPara
   reduce_waves_to_partial<NV, 1>(acc, lds, p.partial + static_cast<int64_t>(blockIdx.x) * p.C, p.C, lane, wave);
 }
 
-// ---- GELU (tanh approximation) ------------------------------------------------------------------------------------
+// ---- pointwise activations: GELU (tanh approximation) and SiLU ------------------------------------------------------
 
 constexpr float kGeluA = 0.7978845608028654f;  // sqrt(2/pi)
 constexpr float kGeluB = 0.044715f;
+enum { kActGelu = 0, kActSilu = 1 };
 
-__device__ __forceinline__ void gelu_eval(float x, float& y, float& dy) {
-  const float x2 = x * x;
-  const float t = tanhf(kGeluA * x * fmaf(kGeluB, x2, 1.f));
-  y = 0.5f * x * (1.f + t);
-  dy = 0.5f * (1.f + t) + 0.5f * x * (1.f - t * t) * kGeluA * fmaf(3.f * kGeluB, x2, 1.f);
+// y = act(x), dy = act'(x)
+template <int ACT>
+__device__ __forceinline__ void act_eval(float x, float& y, float& dy) {
+  if (ACT == kActGelu) {
+    const float x2 = x * x;
+    const float t = tanhf(kGeluA * x * fmaf(kGeluB, x2, 1.f));
+    y = 0.5f * x * (1.f + t);
+    dy = 0.5f * (1.f + t) + 0.5f * x * (1.f - t * t) * kGeluA * fmaf(3.f * kGeluB, x2, 1.f);
+  } else {
+    const float sg = 1.f / (1.f + expf(-x));
+    y = x * sg;
+    dy = sg * fmaf(x, 1.f - sg, 1.f);
+  }
 }
 
-struct GeluParams {
+struct ActParams {
   const void *x, *t;  // t: tangent (forward) or cotangent (backward)
   void *y, *ty;       // backward writes gx to ty
   int64_t total;      // n / 8
-  int bf;
+  int xbf, ybf;       // element types of x (and tx, gx) and of y (and ty, gy)
 };
 
-// MODE 0: y only; 1: y and ty = gelu'(x) * t; 2: ty = gelu'(x) * t only (backward).
-template <int MODE>
-__global__ __launch_bounds__(kThreads) void gelu_kernel(GeluParams p) {
+// MODE 0: y only; 1: y and ty = act'(x) * t; 2: ty = act'(x) * t only (backward, t = gy).
+template <int ACT, int MODE>
+__global__ __launch_bounds__(kThreads) void act_kernel(ActParams p) {
   const int64_t v = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (v >= p.total) return;
   float x[8], t[8], y[8], d[8];
-  load8(p.x, p.bf, v * 8, x);
-  if (MODE) load8(p.t, p.bf, v * 8, t);
+  load8(p.x, p.xbf, v * 8, x);
+  if (MODE) load8(p.t, MODE == 2 ? p.ybf : p.xbf, v * 8, t);
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    gelu_eval(x[e], y[e], d[e]);
+    act_eval<ACT>(x[e], y[e], d[e]);
     if (MODE) d[e] *= t[e];
   }
-  if (MODE != 2) store8(p.y, p.bf, v * 8, y);
-  if (MODE) store8(p.ty, p.bf, v * 8, d);
+  if (MODE != 2) store8(p.y, p.ybf, v * 8, y);
+  if (MODE) store8(p.ty, MODE == 2 ? p.xbf : p.ybf, v * 8, d);
 }
 
 // ---- per-head RMS norm --------------------------------------------------------------------------------------------
@@ -647,6 +656,24 @@ inline int reduce_partials(const float* partial, void* out0, void* out1, int B, 
   return launch_status();
 }
 
+template <int ACT>
+inline int act_impl(const void* x, const void* t, void* y, void* ty, int64_t n, int x_dtype, int y_dtype, int mode,
+                    void* stream) {
+  if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return DMF_ATTN_EDTYPE;
+  if (n < 8 || n % 8 || n / 8 / kThreads + 1 > 0x7fffffffLL) return DMF_ATTN_ESHAPE;
+  if (!x || (mode != 2 && !y) || (mode && (!t || !ty))) return DMF_ATTN_ENULL;
+  if (!aligned16(x) || !aligned16(t) || !aligned16(y) || !aligned16(ty)) return DMF_ATTN_EALIGN;
+  ActParams p{};
+  p.x = x; p.t = t; p.y = y; p.ty = ty; p.total = n / 8;
+  p.xbf = x_dtype == DMF_ATTN_BF16; p.ybf = y_dtype == DMF_ATTN_BF16;
+  const unsigned grid = static_cast<unsigned>((p.total + kThreads - 1) / kThreads);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (mode == 0) hipLaunchKernelGGL((act_kernel<ACT, 0>), dim3(grid), dim3(kThreads), 0, s, p);
+  else if (mode == 1) hipLaunchKernelGGL((act_kernel<ACT, 1>), dim3(grid), dim3(kThreads), 0, s, p);
+  else hipLaunchKernelGGL((act_kernel<ACT, 2>), dim3(grid), dim3(kThreads), 0, s, p);
+  return launch_status();
+}
+
 }  // namespace blk
 }  // namespace dmf
 
@@ -763,28 +790,23 @@ int dmf_gate_residual_bwd(const void* gy, const void* gate, const void* h, void*
   return reduce_partials(workspace, ggate, nullptr, B, p.nchunk, 1, C, p.mbf, s);
 }
 
-static int gelu_impl(const void* x, const void* t, void* y, void* ty, int64_t n, int dtype, int mode, void* stream) {
-  if (!dtype_ok(dtype)) return DMF_ATTN_EDTYPE;
-  if (n < 8 || n % 8 || n / 8 / kThreads + 1 > 0x7fffffffLL) return DMF_ATTN_ESHAPE;
-  if (!x || (mode != 2 && !y) || (mode && (!t || !ty))) return DMF_ATTN_ENULL;
-  if (!aligned16(x) || !aligned16(t) || !aligned16(y) || !aligned16(ty)) return DMF_ATTN_EALIGN;
-  GeluParams p{};
-  p.x = x; p.t = t; p.y = y; p.ty = ty; p.total = n / 8; p.bf = dtype == DMF_ATTN_BF16;
-  const unsigned grid = static_cast<unsigned>((p.total + kThreads - 1) / kThreads);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (mode == 0) hipLaunchKernelGGL(gelu_kernel<0>, dim3(grid), dim3(kThreads), 0, s, p);
-  else if (mode == 1) hipLaunchKernelGGL(gelu_kernel<1>, dim3(grid), dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL(gelu_kernel<2>, dim3(grid), dim3(kThreads), 0, s, p);
-  return launch_status();
-}
-
 int dmf_gelu_tanh_fwd(const void* x, const void* tx, void* y, void* ty, int64_t n, int dtype, void* stream) {
   if (ty && !tx) return DMF_ATTN_ENULL;
-  return gelu_impl(x, tx, y, ty, n, dtype, ty ? 1 : 0, stream);
+  return act_impl<kActGelu>(x, tx, y, ty, n, dtype, dtype, ty ? 1 : 0, stream);
 }
 
 int dmf_gelu_tanh_bwd(const void* gy, const void* x, void* gx, int64_t n, int dtype, void* stream) {
-  return gelu_impl(x, gy, nullptr, gx, n, dtype, 2, stream);
+  return act_impl<kActGelu>(x, gy, nullptr, gx, n, dtype, dtype, 2, stream);
+}
+
+int dmf_silu_fwd(const void* x, const void* tx, void* y, void* ty, int64_t n, int x_dtype, int y_dtype,
+                 void* stream) {
+  if (ty && !tx) return DMF_ATTN_ENULL;
+  return act_impl<kActSilu>(x, tx, y, ty, n, x_dtype, y_dtype, ty ? 1 : 0, stream);
+}
+
+int dmf_silu_bwd(const void* gy, const void* x, void* gx, int64_t n, int x_dtype, int gy_dtype, void* stream) {
+  return act_impl<kActSilu>(x, gy, nullptr, gx, n, x_dtype, gy_dtype, 2, stream);
 }
 
 int dmf_colsum(const void* x, void* out, float* workspace, int64_t rows, int C, int x_dtype, int out_dtype,

@@ -56,6 +56,17 @@ def attn_op(q: Tensor, k: Tensor, v: Tensor, op: str = "base") -> Tensor:
     return x.transpose(1, 2)
 
 
+class SiLU(nn.SiLU):
+    """``nn.SiLU`` (no parameters); one fused primal + tangent kernel when ``block_ops="hip"``."""
+
+    def __init__(self, block_ops: str = "torch"):
+        super().__init__()
+        self.fused = _check_block_ops(block_ops)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return fused.silu(x) if self.fused else super().forward(x)
+
+
 class Linear(nn.Linear):
     """``nn.Linear`` whose forward-mode pass costs one extra GEMM instead of two
     (``block_ops.dual_linear``) when ``block_ops="hip"``; parameters, state-dict
@@ -180,7 +191,7 @@ class DiTBlock(nn.Module):
                               attn_func=block_kwargs.get("attn_func", "base"), block_ops=block_ops)
         self.norm2 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
         self.mlp = Mlp(hidden_size, int(hidden_size * mlp_ratio), block_ops=block_ops)
-        self.adaLN_modulation = nn.Sequential(nn.SiLU(), Linear(hidden_size, 6 * hidden_size, block_ops=block_ops))
+        self.adaLN_modulation = nn.Sequential(SiLU(block_ops), Linear(hidden_size, 6 * hidden_size, block_ops=block_ops))
 
     def forward(self, x: Tensor, c: Tensor) -> Tensor:
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.adaLN_modulation(c).chunk(6, dim=-1)
@@ -200,7 +211,7 @@ class FinalLayer(nn.Module):
         self.fused = _check_block_ops(block_ops)
         self.norm_final = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
         self.linear = Linear(hidden_size, patch_size * patch_size * out_channels, block_ops=block_ops)
-        self.adaLN_modulation = nn.Sequential(nn.SiLU(), Linear(hidden_size, 2 * hidden_size, block_ops=block_ops))
+        self.adaLN_modulation = nn.Sequential(SiLU(block_ops), Linear(hidden_size, 2 * hidden_size, block_ops=block_ops))
 
     def forward(self, x: Tensor, c: Tensor) -> Tensor:
         shift, scale = self.adaLN_modulation(c).chunk(2, dim=-1)

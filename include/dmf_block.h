@@ -9,6 +9,7 @@
  *   - `x + gate * branch`                  models/layers.py:198, 200
  *   - `GELU(approximate="tanh")`           models/layers.py:162
  *   - `RMSNorm` on q and k                 models/layers.py:33-42, 148
+ *   - `SiLU` of the conditioning vector    models/layers.py:185-188, 211-214
  * Every entry point below replaces one such string by a single HBM pass.
  *
  * Conventions
@@ -102,6 +103,20 @@ DMF_ATTN_API int dmf_gelu_tanh_fwd(const void* x, const void* tx, void* y, void*
 
 /* gx = gelu'(x) * gy over n elements (n a multiple of 8). */
 DMF_ATTN_API int dmf_gelu_tanh_bwd(const void* gy, const void* x, void* gx, int64_t n, int dtype, void* stream);
+
+/*
+ * y = x * sigmoid(x) over n elements (n a multiple of 8) and, when `ty` is
+ * given, ty = silu'(x) * tx with silu'(x) = s (1 + x (1 - s)), s = sigmoid(x).
+ * Replaces the `nn.SiLU()` in front of every adaLN projection
+ * (models/layers.py:185-188, 211-214).  x, tx: x_dtype; y, ty: y_dtype (the
+ * conditioning vector is fp32 while the projection that follows wants bf16).
+ */
+DMF_ATTN_API int dmf_silu_fwd(const void* x, const void* tx, void* y, void* ty, int64_t n, int x_dtype, int y_dtype,
+                              void* stream);
+
+/* gx = silu'(x) * gy over n elements; gy: gy_dtype, x and gx: x_dtype. */
+DMF_ATTN_API int dmf_silu_bwd(const void* gy, const void* x, void* gx, int64_t n, int x_dtype, int gy_dtype,
+                              void* stream);
 
 /*
  * Per-head RMS norm over D of a logical (B, L, H, D) tensor:

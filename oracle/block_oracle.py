@@ -18,6 +18,7 @@ independent checks in ``tests/test_block_oracle.py`` pin each function:
 * ``gelu_tanh``      -- pinned: ``torch.nn.functional.gelu(approximate="tanh")``
                         (the reference's ``nn.GELU(approximate="tanh")``,
                         models/layers.py:162) and finite differences for the derivative.
+* ``silu``           -- pinned: ``torch.nn.functional.silu`` and finite differences.
 * ``rms_norm``       -- models/layers.py:33-42 (rounding points included);
                         pinned by the closed form x / sqrt(mean x^2 + eps) * gain, finite
                         differences and the closed-form tangent / gradient
@@ -58,6 +59,11 @@ def gate_residual(x, gate, h):
 def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
     """``nn.GELU(approximate="tanh")`` (models/layers.py:162), written out."""
     return 0.5 * x * (1 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
+
+
+def silu(x: torch.Tensor) -> torch.Tensor:
+    """``nn.SiLU()`` (models/layers.py:186,212), written out."""
+    return x * torch.sigmoid(x)
 
 
 def rms_norm(x: torch.Tensor, gain: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:

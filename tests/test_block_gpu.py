@@ -205,3 +205,23 @@ def test_dual_linear_under_func_jvp_and_autograd():
     _close(xd.grad, gx, 1e-5, "gx")
     _close(wd.grad, gw, 1e-5, "gw")
     _close(bd.grad, gb, 1e-5, "gb")
+
+
+@pytest.mark.parametrize("shape", [(64, 1, 768), (3, 8)])
+@pytest.mark.parametrize("xdt,ydt", [(F32, F32), (F32, BF16), (BF16, BF16)])
+def test_silu_fwd_jvp_bwd(shape, xdt, ydt):
+    print(f"silu {shape} {xdt} {ydt}", flush=True)
+    g = torch.Generator().manual_seed(19)
+    x, t = (2 * torch.randn(*shape, generator=g)).to(xdt), torch.randn(*shape, generator=g).to(xdt)
+    gy = torch.randn(*shape, generator=g).to(ydt)
+    y_ref, ty_ref = bo.jvp(bo.silu, (x.float(),), (t.float(),))
+    y, ty = _lib.silu_fwd(x.to(DEV), t.to(DEV), ydt)
+    assert y.dtype == ydt
+    _close(y, y_ref, _tol(xdt, ydt), "y")
+    _close(ty, ty_ref, _tol(xdt, ydt), "ty")
+    y0, none = _lib.silu_fwd(x.to(DEV), None, ydt)
+    assert none is None and torch.equal(y0, y)
+    (gx_ref,) = bo.grads(bo.silu, (x.float(),), gy.float())
+    gx = _lib.silu_bwd(gy.to(DEV), x.to(DEV))
+    assert gx.dtype == xdt
+    _close(gx, gx_ref, _tol(xdt), "gx")

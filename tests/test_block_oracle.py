@@ -121,3 +121,13 @@ def test_rms_norm_agrees_with_attention_oracle_helper():
     from oracle import attn_oracle as ao
     x = torch.randn(2, 3, 2, 16)
     assert torch.allclose(bo.rms_norm(x, torch.ones(16)), ao.rms_norm(x), atol=1e-6)
+
+
+def test_silu_matches_library_and_derivative():
+    x = torch.linspace(-8, 8, 161, dtype=D64)
+    assert torch.allclose(bo.silu(x), torch.nn.functional.silu(x), atol=1e-14)
+    t = torch.randn(161, dtype=D64)
+    _, ty = bo.jvp(bo.silu, (x,), (t,))
+    assert torch.allclose(ty, _fd(bo.silu, (x,), (t,)), atol=1e-7)
+    s = 1 / (1 + np.exp(-x.numpy()))
+    assert np.allclose(ty.numpy(), s * (1 + x.numpy() * (1 - s)) * t.numpy(), atol=1e-12)
