@@ -13,5 +13,5 @@ All device work is done by hand-written gfx950 kernels reached through the
 C ABI in ``include/dmf_attn.h`` (``dmf_amd/libdmf_attn.so``); there is no
 fallback path: if the library is missing, calls raise.
 """
-from .flash_attention_hip_jvp import FlashAttnFunc, flash_attn_func  # noqa: F401
+from .flash_attention_hip_jvp import FlashAttnFunc, FlashAttnQKVPackedFunc, flash_attn_func, flash_attn_qkvpacked_func  # noqa: F401
 from .layers import attn_op, ATTN_FUNCS  # noqa: F401

@@ -155,16 +155,25 @@ def fwd(q, k, v, scale: float, need_lse: bool = True):
     return o, lse
 
 
-def bwd(dout, q, k, v, o, lse, scale: float):
-    """Backward on the primal output.  Returns (dq, dk, dv), contiguous."""
+def bwd(dout, q, k, v, o, lse, scale: float, out=None):
+    """Backward on the primal output.  Returns (dq, dk, dv): freshly allocated
+    contiguous tensors, or the three tensors given as ``out`` (any (B, L, H, D)
+    views with unit last-dim stride and 16-byte aligned rows, e.g. the three slots
+    of one packed (B, L, 3, H, D) gradient buffer), which the kernels fill in place."""
     _check_inputs(q, k, v, o, dout)
     dout, q, k, v, o = map(_prep, (dout, q, k, v, o))
     lse = _raw(_raw(lse).contiguous())
     B, Lq, H, D = q.shape
     Lkv = k.shape[1]
-    dq = _empty((B, Lq, H, D), q.dtype, q.device)
-    dk = _empty((B, Lkv, H, D), q.dtype, q.device)
-    dv = _empty((B, Lkv, H, D), q.dtype, q.device)
+    if out is None:
+        dq = _empty((B, Lq, H, D), q.dtype, q.device)
+        dk = _empty((B, Lkv, H, D), q.dtype, q.device)
+        dv = _empty((B, Lkv, H, D), q.dtype, q.device)
+    else:
+        dq, dk, dv = map(_raw, out)
+        _check_inputs(q, dq, dk, dv)
+        if dq.shape != q.shape or dk.shape != k.shape or dv.shape != v.shape:
+            raise ValueError("bwd: `out` tensors must have the shapes of q, k, v")
     delta = _empty((B, H, Lq), torch.float32, q.device)
     with torch.cuda.device(q.device):
         rc = load().dmf_attn_bwd(

@@ -557,7 +557,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(RmsParams p) {
 // Work-group (x, y): rows [x*kColsumRows, +kColsumRows), 64 vector columns starting at y*64.  Wave w takes rows
 // w, w+4, ... of the chunk (four loads in flight per lane), the four waves are added through LDS.
 
-constexpr int kColsumRows = 256;
+constexpr int kColsumRows = 64;
 
 struct ColsumParams {
   const void* x;

@@ -107,3 +107,61 @@ def flash_attn_func(q, k, v, softmax_scale=None):
         return fwAD.make_dual(out, t_out)
     out, _, _ = FlashAttnFunc.apply(q, k, v, None, None, None, softmax_scale)
     return out
+
+
+class FlashAttnQKVPackedFunc(torch.autograd.Function):
+    """(qkv, tqkv, softmax_scale) -> (o, lse, to) for a packed (B, L, 3, H, D)
+    projection output -- the buffer ``Attention.forward`` slices q, k, v from
+    (reference models/layers.py:143-147).  Same kernels as ``FlashAttnFunc`` (the
+    slices are read in place); ``backward`` has the kernels write dq, dk, dv into
+    the three slots of one packed gradient buffer, so autograd never has to stack
+    and re-lay-out three separate gradients."""
+
+    @staticmethod
+    def forward(qkv, tqkv, softmax_scale):
+        q, k, v = qkv.unbind(2)
+        scale = _default_scale(q, softmax_scale)
+        if tqkv is not None:
+            o, to, lse = _lib.fwd_jvp(q, k, v, *tqkv.unbind(2), scale)
+        else:
+            o, lse = _lib.fwd(q, k, v, scale, need_lse=True)
+            to = None
+        return o, lse, to
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        qkv, _, softmax_scale = inputs
+        o, lse, _ = outputs
+        ctx.save_for_backward(qkv, o, lse)
+        ctx.save_for_forward(qkv)
+        ctx.softmax_scale = _default_scale(qkv, softmax_scale)
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, dout, *ignored):
+        qkv, o, lse = ctx.saved_tensors
+        if dout is None:
+            return None, None, None
+        gqkv = torch.empty(qkv.shape, dtype=qkv.dtype, device=qkv.device)
+        _lib.bwd(dout, *qkv.unbind(2), o, lse, ctx.softmax_scale, out=gqkv.unbind(2))
+        return gqkv, None, None
+
+    @staticmethod
+    def jvp(ctx, gqkv, *ignored):
+        if gqkv is None:
+            return None, None, None
+        qkv = ctx.saved_tensors[0]
+        q, k, v = _lib._raw(qkv).unbind(2)
+        tq, tk, tv = _lib._raw(gqkv).unbind(2)
+        _, to, _, dlse = _lib.fwd_jvp(q, k, v, tq, tk, tv, ctx.softmax_scale, need_dlse=True)
+        return to, dlse, None
+
+
+def flash_attn_qkvpacked_func(qkv, softmax_scale=None):
+    """Attention on a packed (B, L, 3, H, D) tensor, returns (B, L, H, D); dual in
+    -> dual out, like ``flash_attn_func``."""
+    if qkv.dim() != 5 or qkv.shape[2] != 3:
+        raise ValueError(f"expected a packed (B, L, 3, H, D) tensor, got shape {tuple(qkv.shape)}")
+    p, tg = fwAD.unpack_dual(qkv)
+    out, _, t_out = FlashAttnQKVPackedFunc.apply(p, tg, softmax_scale)
+    return out if tg is None else fwAD.make_dual(out, t_out)

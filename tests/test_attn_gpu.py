@@ -233,3 +233,33 @@ def test_unsupported_head_dim_raises():
         flash_attn_func(q, q, q)
     with pytest.raises(TypeError):
         flash_attn_func(q.half(), q.half(), q.half())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_qkvpacked_func_matches_unpacked_and_writes_packed_grads(dtype):
+    """flash_attn_qkvpacked_func on the (B, L, 3, H, D) projection buffer: same
+    kernels, same bits as flash_attn_func on the three slices; backward fills one
+    packed gradient buffer in place."""
+    import dmf_amd
+    B, L, H, D = 2, 200, 3, 72
+    g = torch.Generator().manual_seed(21)
+    qkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(DEV)
+    tqkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(DEV)
+    dout = torch.randn(B, L, H, D, generator=g).to(dtype).to(DEV)
+    a = qkv.clone().requires_grad_()
+    b = qkv.clone().requires_grad_()
+    o1, to1 = torch.func.jvp(dmf_amd.flash_attn_qkvpacked_func, (a,), (tqkv,))
+    o2, to2 = torch.func.jvp(lambda x: dmf_amd.flash_attn_func(*x.unbind(2)), (b,), (tqkv,))
+    assert torch.equal(o1, o2) and torch.equal(to1, to2)
+    o1.backward(dout)
+    o2.backward(dout)
+    assert a.grad.shape == qkv.shape and torch.equal(a.grad, b.grad)
+    # plain (non-dual, no-grad) call
+    with torch.no_grad():
+        assert torch.equal(dmf_amd.flash_attn_qkvpacked_func(qkv), o1.detach())
+    # dual tensors handed straight to the Function: jvp staticmethod
+    f = lambda x: dmf_amd.FlashAttnQKVPackedFunc.apply(x, None, None)[0]
+    o3, to3 = torch.func.jvp(f, (qkv,), (tqkv,))
+    assert torch.equal(o3, o1.detach()) and torch.equal(to3, to1.detach())
+    with pytest.raises(ValueError):
+        dmf_amd.flash_attn_qkvpacked_func(qkv[:, :, 0])
