@@ -298,9 +298,12 @@ struct ReduceParams {
   int obf;
 };
 
+// Work-group: 64 output vectors (8 columns each); wave w adds chunks w, w+4, ...; the four waves meet in LDS.
 __global__ __launch_bounds__(kThreads) void reduce_partials_kernel(ReduceParams p) {
-  const int64_t v = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (v >= p.total) return;
+  __shared__ float lds[kWaves - 1][64 * 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t v = static_cast<int64_t>(blockIdx.x) * 64 + lane;
+  const bool live = v < p.total;
   const int vec_per_row = p.C / 8;
   const int col = static_cast<int>(v % vec_per_row) * 8;
   const int64_t bk = v / vec_per_row;
@@ -308,14 +311,26 @@ __global__ __launch_bounds__(kThreads) void reduce_partials_kernel(ReduceParams 
   const int64_t b = bk / p.K;
   float s[8];
   zero8(s);
-#pragma unroll 8
-  for (int c = 0; c < p.nchunk; ++c) {
-    float t[8];
-    load8(p.partial, 0, ((b * p.nchunk + c) * p.K + k) * p.C + col, t);
+  if (live) {
+#pragma unroll 4
+    for (int c = wave; c < p.nchunk; c += kWaves) {
+      float t[8];
+      load8(p.partial, 0, ((b * p.nchunk + c) * p.K + k) * p.C + col, t);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) s[e] += t[e];
+      for (int e = 0; e < 8; ++e) s[e] += t[e];
+    }
   }
-  store8(p.out[k], p.obf, b * p.C + col, s);
+  if (wave > 0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) lds[wave - 1][lane * 8 + e] = s[e];
+  }
+  __syncthreads();
+  if (wave == 0 && live) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      for (int w = 0; w < kWaves - 1; ++w) s[e] += lds[w][lane * 8 + e];
+    store8(p.out[k], p.obf, b * p.C + col, s);
+  }
 }
 
 // ---- gated residual -----------------------------------------------------------------------------------------------
@@ -651,7 +666,7 @@ inline int reduce_partials(const float* partial, void* out0, void* out1, int B, 
   r.K = K;
   r.C = C;
   r.obf = obf;
-  const unsigned grid = static_cast<unsigned>((r.total + kThreads - 1) / kThreads);
+  const unsigned grid = static_cast<unsigned>((r.total + 63) / 64);
   hipLaunchKernelGGL(reduce_partials_kernel, dim3(grid), dim3(kThreads), 0, s, r);
   return launch_status();
 }

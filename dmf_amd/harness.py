@@ -104,18 +104,20 @@ def _time(fn, steps: int, warmup: int = 2) -> float:
     return (time.perf_counter() - t0) / steps
 
 
-def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True) -> dict:
+def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=None, variants=None) -> dict:
     """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast, and
     (b) DMFT-XL/2 256px forward+JVP+backward, batch 32.  Variants:
     ``hip_fused_graph`` -- 'hip' attention + fused block glue, replayed as a HIP graph,
     ``hip_fused``       -- the same, launched eagerly from Python,
     ``hip``             -- 'hip' attention inside the reference's tensor expressions,
-    ``base``            -- naive attention (the reference's own CPU-runnable operator)."""
+    ``base``            -- naive attention (the reference's own CPU-runnable operator).
+    ``only`` / ``variants`` restrict the model / the variants that are run."""
     out = {}
-    cases = [("DMFT-B/2", 64, 8, False), ("DMFT-XL/2", 32, 20, True)]
-    variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused", "hip", "hip", False), ("hip", "hip", "torch", False)]
+    cases = [c for c in [("DMFT-B/2", 64, 8, False), ("DMFT-XL/2", 32, 20, True)] if only in (None, c[0])]
+    all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused", "hip", "hip", False), ("hip", "hip", "torch", False)]
     if compare_base:
-        variants.append(("base", "base", "torch", False))
+        all_variants.append(("base", "base", "torch", False))
+    variants = [v for v in all_variants if variants is None or v[0] in variants]
     for name, batch, dmf_depth, train in cases:
         row = {"batch": batch, "mode": "fwd+jvp+bwd" if train else "fwd+jvp", "dtype": "bf16 autocast"}
         data = synthetic_batch(batch, device)
