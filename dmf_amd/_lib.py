@@ -38,6 +38,8 @@ SIGNATURES = {
     "dmf_rmsnorm_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_rmsnorm_bwd": (c_int, [_P] * 6 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_colsum": (c_int, [_P] * 3 + [_L, _I, _I, _I, _P]),
+    "dmf_residual_ln_modulate_fwd": (c_int, [_P] * 14 + [_S] + [_I] * 3 + [_F] + [_I] * 4 + [_P]),
+    "dmf_residual_ln_modulate_bwd": (c_int, [_P] * 12 + [_L, _L] + [_I] * 3 + [_F] + [_I] * 4 + [_P]),
     "dmf_silu_fwd": (c_int, [_P] * 4 + [_L, _I, _I, _P]),
     "dmf_silu_bwd": (c_int, [_P] * 3 + [_L, _I, _I, _P]),
 }
@@ -400,3 +402,49 @@ def silu_bwd(gy, x):
         rc = load().dmf_silu_bwd(gy.data_ptr(), x.data_ptr(), gx.data_ptr(), x.numel(), _dtype_code(x), _dtype_code(gy), _stream(x))
     _check(rc, "dmf_silu_bwd")
     return gx
+
+
+def residual_ln_modulate_fwd(x, gate, h, shift, scale, tx=None, tgate=None, th=None, tshift=None, tscale=None,
+                             eps: float = 1e-6, out_dtype=None, jvp=False):
+    """(y, z, ty, tz): y = x + gate*h (dtype of x), z = LayerNorm(y)*(1+scale)+shift
+    (``out_dtype``); the tangents are None unless ``jvp``."""
+    B, L, C = _blc(x)
+    _same_dtype("residual_ln_modulate x", x, tx)
+    _same_dtype("residual_ln_modulate h", h, th)
+    _same_dtype("residual_ln_modulate modulation", gate, tgate, shift, scale, tshift, tscale)
+    if h.shape != x.shape:
+        raise ValueError("residual_ln_modulate: x and h must have the same shape")
+    x, tx, h, th = _dense(x), _dense(tx), _dense(h), _dense(th)
+    mods = [_mod(t, B, C) for t in (gate, tgate, shift, scale, tshift, tscale)]
+    out_dtype = out_dtype or x.dtype
+    y = _empty((B, L, C), x.dtype, x.device)
+    z = _empty((B, L, C), out_dtype, x.device)
+    ty = _empty((B, L, C), x.dtype, x.device) if jvp else None
+    tz = _empty((B, L, C), out_dtype, x.device) if jvp else None
+    with torch.cuda.device(x.device):
+        rc = load().dmf_residual_ln_modulate_fwd(
+            x.data_ptr(), _ptr(tx), mods[0][0].data_ptr(), _ptr(mods[1][0]), h.data_ptr(), _ptr(th),
+            mods[2][0].data_ptr(), mods[3][0].data_ptr(), _ptr(mods[4][0]), _ptr(mods[5][0]),
+            y.data_ptr(), _ptr(ty), z.data_ptr(), _ptr(tz), (c_int64 * 6)(*[m[1] for m in mods]), B, L, C, float(eps),
+            _dtype_code(x), _dtype_code(mods[0][0]), _dtype_code(h), _dtype_code(z), _stream(x))
+    _check(rc, "dmf_residual_ln_modulate_fwd")
+    return y, z, ty, tz
+
+
+def residual_ln_modulate_bwd(gy, gz, y, h, gate, scale, eps: float = 1e-6):
+    """(gx, gh, ggate, gshift, gscale); ``gy`` may be None."""
+    B, L, C = _blc(y)
+    gy, gz, y, h = _dense(gy), _dense(gz), _dense(y), _dense(h)
+    gate, gs = _mod(gate, B, C)
+    scale, ss = _mod(scale, B, C)
+    gx = _empty((B, L, C), y.dtype, y.device)
+    gh = _empty((B, L, C), h.dtype, y.device)
+    ggate, gshift, gscale = (_empty((B, C), gate.dtype, y.device) for _ in range(3))
+    ws = _workspace(4, B, L, C, y.device)
+    with torch.cuda.device(y.device):
+        rc = load().dmf_residual_ln_modulate_bwd(
+            _ptr(gy), gz.data_ptr(), y.data_ptr(), h.data_ptr(), gate.data_ptr(), scale.data_ptr(), gx.data_ptr(), gh.data_ptr(),
+            ggate.data_ptr(), gshift.data_ptr(), gscale.data_ptr(), ws.data_ptr(), gs, ss, B, L, C, float(eps),
+            _dtype_code(y), _dtype_code(gate), _dtype_code(h), _dtype_code(gz), _stream(y))
+    _check(rc, "dmf_residual_ln_modulate_bwd")
+    return gx, gh, ggate, gshift, gscale

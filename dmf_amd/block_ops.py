@@ -5,6 +5,7 @@ attention operator in the reference's block (models/layers.py):
 
 * ``ln_modulate(x, shift, scale)``  = ``modulate(LayerNorm(x), shift, scale)``   (:28-29, :198, :200, :219)
 * ``gate_residual(x, gate, h)``     = ``x + gate * h``                           (:198, :200)
+* ``residual_ln_modulate(x, gate, h, shift, scale)`` = the two above back to back (:198-200)
 * ``gelu_tanh(x)``                  = ``nn.GELU(approximate="tanh")(x)``         (:162, :166)
 * ``rms_norm(x, gain)``             = ``RMSNorm.forward``                        (:33-42, :148)
 * ``silu(x)``                       = ``nn.SiLU()`` of the adaLN branch          (:185-188, :211-214)
@@ -86,6 +87,32 @@ class GateResidualFunc(torch.autograd.Function):
         gate, h = ctx.saved_tensors
         gh, ggate = _lib.gate_residual_bwd(gy, gate, h)
         return gy, _like(ggate, ctx.gate_shape), gh, None, None, None, None
+
+
+class ResidualLNModulateFunc(torch.autograd.Function):
+    """(x, gate, h, shift, scale, tx, tgate, th, tshift, tscale, eps, out_dtype, jvp) -> (y, z, ty, tz)."""
+
+    @staticmethod
+    def forward(x, gate, h, shift, scale, tx, tgate, th, tshift, tscale, eps, out_dtype, jvp):
+        return _lib.residual_ln_modulate_fwd(x, gate, h, shift, scale, tx, tgate, th, tshift, tscale, eps, out_dtype, jvp)
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        x, gate, h, shift, scale = inputs[:5]
+        ctx.save_for_backward(outputs[0], h, gate, scale)
+        ctx.eps, ctx.shapes = inputs[10], (gate.shape, shift.shape, scale.shape)
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, gy, gz, gty, gtz):
+        if gy is None and gz is None:
+            return (None,) * 13
+        y, h, gate, scale = ctx.saved_tensors
+        if gz is None:   # only the residual output was used
+            gh, ggate = _lib.gate_residual_bwd(gy, gate, h)
+            return (gy, _like(ggate, ctx.shapes[0]), gh) + (None,) * 10
+        gx, gh, ggate, gshift, gscale = _lib.residual_ln_modulate_bwd(gy, gz, y, h, gate, scale, ctx.eps)
+        return (gx, _like(ggate, ctx.shapes[0]), gh, _like(gshift, ctx.shapes[1]), _like(gscale, ctx.shapes[2])) + (None,) * 8
 
 
 class GeluTanhFunc(torch.autograd.Function):
@@ -235,6 +262,17 @@ def gate_residual(x, gate, h):
         xp, tx = xp.to(dt), (None if tx is None else tx.to(dt))
     y, ty = GateResidualFunc.apply(xp, gp, hp, tx, tg, th, dual)
     return fwAD.make_dual(y, ty) if dual else y
+
+
+def residual_ln_modulate(x, gate, h, shift, scale, eps: float = 1e-6):
+    """``y = x + gate * h`` and ``z = LayerNorm(y) * (1 + scale) + shift`` in one pass;
+    returns ``(y, z)`` with the dtypes ``gate_residual`` and ``ln_modulate`` would give."""
+    (xp, gp, hp, shp, scp), (tx, tg, th, tsh, tsc), dual = _unpack(x, gate, h, shift, scale)
+    dt = torch.promote_types(xp.dtype, hp.dtype)
+    if xp.dtype != dt:
+        xp, tx = xp.to(dt), (None if tx is None else tx.to(dt))
+    y, z, ty, tz = ResidualLNModulateFunc.apply(xp, gp, hp, shp, scp, tx, tg, th, tsh, tsc, eps, _autocast_dtype(xp), dual)
+    return (fwAD.make_dual(y, ty), fwAD.make_dual(z, tz)) if dual else (y, z)
 
 
 def gelu_tanh(x):

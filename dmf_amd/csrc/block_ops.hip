@@ -70,17 +70,27 @@ __device__ __forceinline__ float sum8(const float (&v)[8]) {
   return ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
+// v + (v rotated right by N lanes within each row of 16 lanes), as one DPP-modified add
+template <int N>
+__device__ __forceinline__ float row_ror_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, false));
 }
 
-// sum over the 16 lanes of an aligned lane group
+// sum over the 16 lanes of an aligned lane group; every lane of the group gets the same bits
 __device__ __forceinline__ float group16_sum(float v) {
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
+  v = row_ror_add<8>(v);
+  v = row_ror_add<4>(v);
+  v = row_ror_add<2>(v);
+  return row_ror_add<1>(v);
+}
+
+// sum over the wave; every lane gets the same bits (no LDS traffic: DPP rotations inside the rows of 16 lanes, then the
+// 16- and 32-lane swaps)
+__device__ __forceinline__ float wave_sum(float v) {
+  v = group16_sum(v);
+  float even, odd;
+  swap16f(v, even, odd);
+  return xhalf_sum(even + odd);
 }
 
 // ---- a row of C elements held by one wave: lane owns columns (j*64 + lane)*8 .. +8, j < NV -------------------------
@@ -292,7 +302,7 @@ __global__ __launch_bounds__(kThreads) void ln_modulate_bwd_kernel(LnBwdParams p
 // out[k][b][c] = sum_chunk partial[b][chunk][k][c]; out[k] dense (B, C) of the given element type.
 struct ReduceParams {
   const float* partial;
-  void* out[2];
+  void* out[3];
   int64_t total;  // B * K * C / 8 vectors
   int nchunk, K, C;
   int obf;
@@ -403,6 +413,139 @@ __global__ __launch_bounds__(kThreads) void gate_residual_bwd_kernel(GateBwdPara
     store_row(p.gh, p.hbf, base, p.C, lane, g);
   }
   reduce_waves_to_partial<NV, 1>(acc, lds, p.partial + static_cast<int64_t>(blockIdx.x) * p.C, p.C, lane, wave);
+}
+
+// ---- gated residual fused with the LayerNorm + modulate that consumes it ---------------------------------------------
+// y = x + gate * h;  z = LayerNorm(y) * (1 + scale) + shift  (and tangents): the residual stream is read once and
+// written once per half block instead of being re-read by a separate normalisation kernel.
+
+struct ResLnFwdParams {
+  const void *x, *tx, *gate, *tgate, *h, *th, *shift, *scale, *tshift, *tscale;
+  void *y, *ty, *z, *tz;
+  int64_t rows, ms[6];  // batch strides of gate, tgate, shift, scale, tshift, tscale
+  int L, C;
+  float eps;
+  int xbf, mbf, hbf, zbf;
+};
+
+template <int NV, bool JVP>
+__global__ __launch_bounds__(kThreads) void residual_ln_modulate_fwd_kernel(ResLnFwdParams p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
+  if (row >= p.rows) return;  // no work-group barrier in this kernel
+  const int64_t b = row / p.L, base = row * p.C;
+  Row<NV> y, t, h;
+  load_row(p.x, p.xbf, base, p.C, lane, y);
+  load_row(p.h, p.hbf, base, p.C, lane, h);
+  if (JVP) load_row(p.tx, p.xbf, base, p.C, lane, t);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int col = (j * 64 + lane) * 8;
+    if (col >= p.C) continue;
+    float g[8];
+    load8(p.gate, p.mbf, b * p.ms[0] + col, g);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y.v[j][e] = fmaf(g[e], h.v[j][e], y.v[j][e]);
+    store8(p.y, p.xbf, base + col, y.v[j]);
+    if (JVP) {
+      float tg[8], th[8];
+      load8(p.tgate, p.mbf, b * p.ms[1] + col, tg);
+      load8(p.th, p.hbf, base + col, th);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t.v[j][e] = fmaf(tg[e], h.v[j][e], fmaf(g[e], th[e], t.v[j][e]));
+      store8(p.ty, p.xbf, base + col, t.v[j]);
+    }
+  }
+  const float rstd = normalize_row(y, p.C, lane, p.eps);
+  if (JVP) project_row(t, y, rstd, p.C, lane);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int col = (j * 64 + lane) * 8;
+    if (col >= p.C) continue;
+    float sh[8], sc[8], out[8];
+    load8(p.shift, p.mbf, b * p.ms[2] + col, sh);
+    load8(p.scale, p.mbf, b * p.ms[3] + col, sc);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = fmaf(y.v[j][e], 1.f + sc[e], sh[e]);
+    store8(p.z, p.zbf, base + col, out);
+    if (JVP) {
+      float tsh[8], tsc[8];
+      load8(p.tshift, p.mbf, b * p.ms[4] + col, tsh);
+      load8(p.tscale, p.mbf, b * p.ms[5] + col, tsc);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = fmaf(t.v[j][e], 1.f + sc[e], fmaf(y.v[j][e], tsc[e], tsh[e]));
+      store8(p.tz, p.zbf, base + col, out);
+    }
+  }
+}
+
+struct ResLnBwdParams {
+  const void *gy, *gz, *y, *h, *gate, *scale;  // gy may be NULL (no other consumer of y)
+  void *gx, *gh;
+  float* partial;  // (B, nchunk, 3, C): [0] sum g*h (gate), [1] sum gz (shift), [2] sum gz*yh (scale)
+  int64_t gs, ss;
+  int L, C, nchunk;
+  float eps;
+  int xbf, mbf, hbf, zbf;
+};
+
+template <int NV>
+__global__ __launch_bounds__(kThreads) void residual_ln_modulate_bwd_kernel(ResLnBwdParams p) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t b = blockIdx.x / p.nchunk;
+  const int chunk = blockIdx.x % p.nchunk;
+  const int r1 = min(p.L, (chunk + 1) * kChunkRows);
+  Row<NV> one_plus_scale, gate, acc[3];
+  load_row(p.scale, p.mbf, b * p.ss, p.C, lane, one_plus_scale);
+  load_row(p.gate, p.mbf, b * p.gs, p.C, lane, gate);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    zero8(acc[0].v[j]);
+    zero8(acc[1].v[j]);
+    zero8(acc[2].v[j]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) one_plus_scale.v[j][e] += 1.f;
+  }
+  for (int r = chunk * kChunkRows + wave; r < r1; r += kWaves) {
+    const int64_t base = (b * p.L + r) * p.C;
+    Row<NV> yh, g, o;
+    load_row(p.y, p.xbf, base, p.C, lane, yh);
+    load_row(p.gz, p.zbf, base, p.C, lane, g);
+    const float rstd = normalize_row(yh, p.C, lane, p.eps);
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        acc[1].v[j][e] += g.v[j][e];
+        acc[2].v[j][e] = fmaf(g.v[j][e], yh.v[j][e], acc[2].v[j][e]);
+        g.v[j][e] *= one_plus_scale.v[j][e];
+      }
+    project_row(g, yh, rstd, p.C, lane);
+    load_row(p.gy, p.xbf, base, p.C, lane, o);   // NULL reads as zeros
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g.v[j][e] += o.v[j][e];
+    store_row(p.gx, p.xbf, base, p.C, lane, g);
+    load_row(p.h, p.hbf, base, p.C, lane, o);
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        acc[0].v[j][e] = fmaf(g.v[j][e], o.v[j][e], acc[0].v[j][e]);
+        g.v[j][e] *= gate.v[j][e];
+      }
+    store_row(p.gh, p.hbf, base, p.C, lane, g);
+  }
+  // one accumulator at a time through the same LDS slab
+  float* out = p.partial + static_cast<int64_t>(blockIdx.x) * 3 * p.C;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    Row<NV> one[1] = {acc[k]};
+    reduce_waves_to_partial<NV, 1>(one, lds, out + static_cast<int64_t>(k) * p.C, p.C, lane, wave);
+    __syncthreads();
+  }
 }
 
 // ---- pointwise activations: GELU (tanh approximation) and SiLU ------------------------------------------------------
@@ -656,11 +799,12 @@ inline int dispatch_nv(int C, F&& f) {
 }
 
 inline int reduce_partials(const float* partial, void* out0, void* out1, int B, int nchunk, int K, int C, int obf,
-                           hipStream_t s) {
+                           hipStream_t s, void* out2 = nullptr) {
   ReduceParams r{};
   r.partial = partial;
   r.out[0] = out0;
   r.out[1] = out1;
+  r.out[2] = out2;
   r.total = static_cast<int64_t>(B) * K * (C / 8);
   r.nchunk = nchunk;
   r.K = K;
@@ -703,6 +847,7 @@ int64_t dmf_block_workspace_floats(int which, int B, int L, int dim) {
     case 1: return static_cast<int64_t>(B) * nchunks(L) * dim;
     case 2: return static_cast<int64_t>(kRmsBlocksMax) * dim;
     case 3: return ((static_cast<int64_t>(B) * L + kColsumRows - 1) / kColsumRows) * dim;
+    case 4: return static_cast<int64_t>(B) * nchunks(L) * 3 * dim;
     default: return 0;
   }
 }
@@ -803,6 +948,70 @@ int dmf_gate_residual_bwd(const void* gy, const void* gate, const void* h, void*
   });
   if (rc) return rc;
   return reduce_partials(workspace, ggate, nullptr, B, p.nchunk, 1, C, p.mbf, s);
+}
+
+int dmf_residual_ln_modulate_fwd(const void* x, const void* tx, const void* gate, const void* tgate, const void* h,
+                                 const void* th, const void* shift, const void* scale, const void* tshift,
+                                 const void* tscale, void* y, void* ty, void* z, void* tz, const int64_t* mod_strides,
+                                 int B, int L, int C, float eps, int x_dtype, int mod_dtype, int h_dtype, int z_dtype,
+                                 void* stream) {
+  if (!dtype_ok(x_dtype) || !dtype_ok(mod_dtype) || !dtype_ok(h_dtype) || !dtype_ok(z_dtype)) return DMF_ATTN_EDTYPE;
+  if (int rc = check_blc(B, L, C)) return rc;
+  if (!x || !gate || !h || !shift || !scale || !y || !z || !mod_strides) return DMF_ATTN_ENULL;
+  const bool jvp = ty != nullptr || tz != nullptr;
+  if (jvp && (!ty || !tz)) return DMF_ATTN_ENULL;
+  if (!aligned16(x) || !aligned16(tx) || !aligned16(h) || !aligned16(th) || !aligned16(y) || !aligned16(ty) ||
+      !aligned16(z) || !aligned16(tz))
+    return DMF_ATTN_EALIGN;
+  const void* mods[6] = {gate, tgate, shift, scale, tshift, tscale};
+  const bool required[6] = {true, false, true, true, false, false};
+  for (int i = 0; i < 6; ++i)
+    if (int rc = check_mod(mods[i], mod_strides[i], mod_dtype, required[i])) return rc;
+  ResLnFwdParams p{};
+  p.x = x; p.tx = tx; p.gate = gate; p.tgate = tgate; p.h = h; p.th = th;
+  p.shift = shift; p.scale = scale; p.tshift = tshift; p.tscale = tscale;
+  p.y = y; p.ty = ty; p.z = z; p.tz = tz;
+  p.rows = static_cast<int64_t>(B) * L;
+  for (int i = 0; i < 6; ++i) p.ms[i] = mod_strides[i];
+  p.L = L; p.C = C; p.eps = eps;
+  p.xbf = x_dtype == DMF_ATTN_BF16; p.mbf = mod_dtype == DMF_ATTN_BF16;
+  p.hbf = h_dtype == DMF_ATTN_BF16; p.zbf = z_dtype == DMF_ATTN_BF16;
+  const unsigned grid = static_cast<unsigned>((p.rows + kWaves - 1) / kWaves);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return dispatch_nv(C, [&](auto nv) {
+    constexpr int NV = decltype(nv)::value;
+    if (jvp) hipLaunchKernelGGL((residual_ln_modulate_fwd_kernel<NV, true>), dim3(grid), dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((residual_ln_modulate_fwd_kernel<NV, false>), dim3(grid), dim3(kThreads), 0, s, p);
+  });
+}
+
+int dmf_residual_ln_modulate_bwd(const void* gy, const void* gz, const void* y, const void* h, const void* gate,
+                                 const void* scale, void* gx, void* gh, void* ggate, void* gshift, void* gscale,
+                                 float* workspace, int64_t gate_stride, int64_t scale_stride, int B, int L, int C,
+                                 float eps, int x_dtype, int mod_dtype, int h_dtype, int z_dtype, void* stream) {
+  if (!dtype_ok(x_dtype) || !dtype_ok(mod_dtype) || !dtype_ok(h_dtype) || !dtype_ok(z_dtype)) return DMF_ATTN_EDTYPE;
+  if (int rc = check_blc(B, L, C)) return rc;
+  if (!gz || !y || !h || !gate || !scale || !gx || !gh || !ggate || !gshift || !gscale || !workspace) return DMF_ATTN_ENULL;
+  if (!aligned16(gy) || !aligned16(gz) || !aligned16(y) || !aligned16(h) || !aligned16(gx) || !aligned16(gh) ||
+      !aligned16(ggate) || !aligned16(gshift) || !aligned16(gscale) || !aligned16(workspace))
+    return DMF_ATTN_EALIGN;
+  if (int rc = check_mod(gate, gate_stride, mod_dtype, true)) return rc;
+  if (int rc = check_mod(scale, scale_stride, mod_dtype, true)) return rc;
+  ResLnBwdParams p{};
+  p.gy = gy; p.gz = gz; p.y = y; p.h = h; p.gate = gate; p.scale = scale; p.gx = gx; p.gh = gh;
+  p.partial = workspace; p.gs = gate_stride; p.ss = scale_stride;
+  p.L = L; p.C = C; p.nchunk = nchunks(L); p.eps = eps;
+  p.xbf = x_dtype == DMF_ATTN_BF16; p.mbf = mod_dtype == DMF_ATTN_BF16;
+  p.hbf = h_dtype == DMF_ATTN_BF16; p.zbf = z_dtype == DMF_ATTN_BF16;
+  const unsigned grid = static_cast<unsigned>(B) * p.nchunk;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int rc = dispatch_nv(C, [&](auto nv) {
+    constexpr int NV = decltype(nv)::value;
+    constexpr size_t lds = (kWaves - 1) * NV * 512 * sizeof(float);
+    hipLaunchKernelGGL((residual_ln_modulate_bwd_kernel<NV>), dim3(grid), dim3(kThreads), lds, s, p);
+  });
+  if (rc) return rc;
+  return reduce_partials(workspace, ggate, gshift, B, p.nchunk, 3, C, p.mbf, s, gscale);
 }
 
 int dmf_gelu_tanh_fwd(const void* x, const void* tx, void* y, void* ty, int64_t n, int dtype, void* stream) {

@@ -58,6 +58,7 @@ class DMFT(nn.Module):
         self.in_channels = self.out_channels = in_channels
         self.num_heads, self.num_classes = num_heads, num_classes
         self.dmf_depth, self.use_logvar = dmf_depth, use_logvar
+        self.fused = _check_block_ops(block_kwargs.get("block_ops", "torch"))
 
         self.x_embedder = PatchEmbed(input_size, patch_size, in_channels, hidden_size, bias=True,
                                      block_ops=block_kwargs.get("block_ops", "torch"))
@@ -128,6 +129,24 @@ class DMFT(nn.Module):
         x = torch.einsum("nhwpqc->nchpwq", x)
         return x.reshape(x.shape[0], c, h * p, w * p)
 
+    def _forward_chained(self, x, c_t, c_r):
+        """The block stack and final layer in fused mode: same values as the plain
+        loop, but every gated residual is computed by the kernel that also
+        normalises and modulates the result for its consumer (the block's own MLP
+        branch, the next block's attention branch, or the final layer), so the
+        residual stream is read and written once per half block."""
+        conds = [c_t] * self.dmf_depth + [c_r] * (len(self.blocks) - self.dmf_depth)
+        mods = [blk.adaLN_modulation(c).chunk(6, dim=-1) for blk, c in zip(self.blocks, conds)]
+        f_shift, f_scale = self.final_layer.adaLN_modulation(c_r).chunk(2, dim=-1)
+        z = block_ops_mod.ln_modulate(x, mods[0][0], mods[0][1], self.blocks[0].norm1.eps)
+        for i, blk in enumerate(self.blocks):
+            if i + 1 < len(self.blocks):
+                nxt = (mods[i + 1][0], mods[i + 1][1], self.blocks[i + 1].norm1.eps)
+            else:
+                nxt = (f_shift, f_scale, self.final_layer.norm_final.eps)
+            x, z = blk.forward_chained(x, z, mods[i], *nxt)
+        return self.final_layer.linear(z)
+
     def forward(self, x, t, r, y, return_logvar: bool = False):
         t, r = t.reshape(-1), r.reshape(-1)
         x = self.x_embedder(x) + self.pos_embed
@@ -135,12 +154,15 @@ class DMFT(nn.Module):
         t_embed = self.t_embedder(t).reshape(B, -1, D)
         y_embed = self.y_embedder(y).reshape(B, -1, D)
         c_t = t_embed + y_embed
-        for block in self.blocks[:self.dmf_depth]:      # encoder: conditioned on t
-            x = block(x, c_t)
-        c_r = self.t_embedder(r).reshape(B, -1, D) + y_embed
-        for block in self.blocks[self.dmf_depth:]:      # decoder: conditioned on r
-            x = block(x, c_r)
-        x = self.unpatchify(self.final_layer(x, c_r))
+        if self.fused:
+            x = self.unpatchify(self._forward_chained(x, c_t, self.t_embedder(r).reshape(B, -1, D) + y_embed))
+        else:
+            for block in self.blocks[:self.dmf_depth]:      # encoder: conditioned on t
+                x = block(x, c_t)
+            c_r = self.t_embedder(r).reshape(B, -1, D) + y_embed
+            for block in self.blocks[self.dmf_depth:]:      # decoder: conditioned on r
+                x = block(x, c_r)
+            x = self.unpatchify(self.final_layer(x, c_r))
         if return_logvar:
             logvar = self.logvar_linear(torch.cat([self.logvar_t_embedder(t), self.logvar_t_embedder(r)], dim=1))
             return x, logvar.view(-1, *[1] * (x.ndim - 1))

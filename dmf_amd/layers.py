@@ -201,12 +201,25 @@ class DiTBlock(nn.Module):
 
     def forward(self, x: Tensor, c: Tensor) -> Tensor:
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.adaLN_modulation(c).chunk(6, dim=-1)
-        if self.fused:   # same expressions, each norm+modulate and each gated residual in one kernel
-            x = fused.gate_residual(x, gate_msa, self.attn(fused.ln_modulate(x, shift_msa, scale_msa, self.norm1.eps)))
-            return fused.gate_residual(x, gate_mlp, self.mlp(fused.ln_modulate(x, shift_mlp, scale_mlp, self.norm2.eps)))
+        if self.fused:   # same expressions; the first residual is fused with the norm+modulate that follows it
+            x, z = fused.residual_ln_modulate(x, gate_msa, self.attn(fused.ln_modulate(x, shift_msa, scale_msa, self.norm1.eps)),
+                                              shift_mlp, scale_mlp, self.norm2.eps)
+            return fused.gate_residual(x, gate_mlp, self.mlp(z))
         x = x + gate_msa * self.attn(modulate(self.norm1(x), shift_msa, scale_msa))
         x = x + gate_mlp * self.mlp(modulate(self.norm2(x), shift_mlp, scale_mlp))
         return x
+
+    def forward_chained(self, x: Tensor, z: Tensor, mods, next_shift: Tensor, next_scale: Tensor, next_eps: float):
+        """Fused-mode variant for a stack of blocks.  ``z`` is this block's already
+        normalised and modulated input (``modulate(norm1(x), shift_msa, scale_msa)``,
+        produced by the previous block's last kernel), ``mods`` the six chunks of
+        ``self.adaLN_modulation(c)``; the block's second residual is fused with the
+        *next* consumer's norm + modulate (``next_shift`` / ``next_scale``: the next
+        block's msa pair, or the final layer's).  Returns ``(x_out, z_next)``; same
+        values as ``forward``."""
+        _, _, gate_msa, shift_mlp, scale_mlp, gate_mlp = mods
+        x, z = fused.residual_ln_modulate(x, gate_msa, self.attn(z), shift_mlp, scale_mlp, self.norm2.eps)
+        return fused.residual_ln_modulate(x, gate_mlp, self.mlp(z), next_shift, next_scale, next_eps)
 
 
 class FinalLayer(nn.Module):

@@ -41,7 +41,8 @@ extern "C" {
 
 /* Number of fp32 workspace elements a backward entry point needs.
  * `which`: 0 = dmf_ln_modulate_bwd, 1 = dmf_gate_residual_bwd (rows = B*L, dim = C),
- *          2 = dmf_rmsnorm_bwd (dim = D; B, L ignored), 3 = dmf_colsum (rows = B*L, dim = C).
+ *          2 = dmf_rmsnorm_bwd (dim = D; B, L ignored), 3 = dmf_colsum (rows = B*L, dim = C),
+ *          4 = dmf_residual_ln_modulate_bwd (rows = B*L, dim = C).
  * Returns 0 on bad input. */
 DMF_ATTN_API int64_t dmf_block_workspace_floats(int which, int B, int L, int dim);
 
@@ -92,6 +93,36 @@ DMF_ATTN_API int dmf_gate_residual_fwd(const void* x, const void* tx, const void
 DMF_ATTN_API int dmf_gate_residual_bwd(const void* gy, const void* gate, const void* h, void* gh, void* ggate,
                                        float* workspace, int64_t gate_stride, int B, int L, int C,
                                        int gy_dtype, int mod_dtype, int h_dtype, void* stream);
+
+/*
+ * The gated residual and the LayerNorm + modulate that consumes its result, in
+ * one pass over the residual stream (`x = x + gate_msa * attn(...)` followed by
+ * `modulate(self.norm2(x), shift_mlp, scale_mlp)`, models/layers.py:198-200, and
+ * likewise across the block boundary, :200 -> next block's :198, or :219):
+ *   y = x + gate * h,  z = LayerNorm(y) * (1 + scale) + shift,
+ * with ty, tz as in the two separate entry points when ty and tz are given
+ * (both or neither).  x, tx, y, ty: x_dtype; h, th: h_dtype; z, tz: z_dtype;
+ * gate, tgate, shift, scale, tshift, tscale: (B, C) of mod_dtype with batch
+ * strides mod_strides[0..5] in that order.
+ */
+DMF_ATTN_API int dmf_residual_ln_modulate_fwd(const void* x, const void* tx, const void* gate, const void* tgate,
+                                              const void* h, const void* th, const void* shift, const void* scale,
+                                              const void* tshift, const void* tscale, void* y, void* ty, void* z,
+                                              void* tz, const int64_t* mod_strides, int B, int L, int C, float eps,
+                                              int x_dtype, int mod_dtype, int h_dtype, int z_dtype, void* stream);
+
+/*
+ * Backward of the primal of dmf_residual_ln_modulate_fwd.  gy (x_dtype, may be
+ * NULL) is the gradient reaching y from its other consumers, gz (z_dtype) the
+ * gradient of z:  g = gy + LayerNorm-backward(gz * (1 + scale); y),
+ *   gx = g (x_dtype),  gh = gate * g (h_dtype),  ggate = sum_l g * h,
+ *   gshift = sum_l gz,  gscale = sum_l gz * yh   (dense (B, C) of mod_dtype).
+ */
+DMF_ATTN_API int dmf_residual_ln_modulate_bwd(const void* gy, const void* gz, const void* y, const void* h,
+                                              const void* gate, const void* scale, void* gx, void* gh, void* ggate,
+                                              void* gshift, void* gscale, float* workspace, int64_t gate_stride,
+                                              int64_t scale_stride, int B, int L, int C, float eps, int x_dtype,
+                                              int mod_dtype, int h_dtype, int z_dtype, void* stream);
 
 /*
  * y = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) over n elements and,
