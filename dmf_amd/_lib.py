@@ -12,6 +12,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 
 import torch
 from torch._C import _functorch
+from torch._functorch.pyfunctorch import retrieve_all_functorch_interpreters as _interpreters
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdmf_attn.so")
@@ -84,6 +85,20 @@ def _raw(t):
     while t is not None and _functorch.is_functorch_wrapped_tensor(t):
         t = _functorch.get_unwrapped(t)
     return t
+
+
+def run_function(fn_cls, *args):
+    """``fn_cls.apply(*args)`` -- or, when nothing needs a gradient and no functorch
+    transform other than ``jvp`` is active, ``fn_cls.forward(*args)`` directly.  The
+    operators of this package unpack forward-AD duals themselves, so the only thing
+    ``apply`` adds then is the (considerable) per-call cost of building an autograd
+    node through functorch's custom-Function dispatch."""
+    # (inside a functorch level the wrapper tensors do not report requires_grad; the wrapped values do)
+    needs_grad = torch.is_grad_enabled() and any(isinstance(a, torch.Tensor) and (a.requires_grad or _raw(a).requires_grad)
+                                                 for a in args)
+    if not needs_grad and all(i.key() == _functorch.TransformType.Jvp for i in _interpreters()):
+        return fn_cls.forward(*args)
+    return fn_cls.apply(*args)
 
 
 def _empty(shape, dtype, device) -> torch.Tensor:

@@ -233,7 +233,7 @@ def dual_linear(x, weight, bias=None):
     """``F.linear(x, weight, bias)``; a forward-AD dual ``x`` gives a dual result
     (weight and bias are constants of the tangent map)."""
     (xp,), (tx,), dual = _unpack(x)
-    y, ty, _ = DualLinearFunc.apply(xp, tx, weight, bias)
+    y, ty, _ = _lib.run_function(DualLinearFunc, xp, tx, weight, bias)
     return fwAD.make_dual(y, ty) if dual else y
 
 
@@ -249,7 +249,7 @@ def ln_modulate(x, shift, scale, eps: float = 1e-6):
     autocast the result is produced directly in the autocast dtype (it only ever
     feeds a Linear, which would cast it)."""
     (xp, shp, scp), (tx, tsh, tsc), dual = _unpack(x, shift, scale)
-    y, ty = LNModulateFunc.apply(xp, shp, scp, tx, tsh, tsc, eps, _autocast_dtype(xp), dual)
+    y, ty = _lib.run_function(LNModulateFunc, xp, shp, scp, tx, tsh, tsc, eps, _autocast_dtype(xp), dual)
     return fwAD.make_dual(y, ty) if dual else y
 
 
@@ -260,7 +260,7 @@ def gate_residual(x, gate, h):
     dt = torch.promote_types(xp.dtype, hp.dtype)
     if xp.dtype != dt:
         xp, tx = xp.to(dt), (None if tx is None else tx.to(dt))
-    y, ty = GateResidualFunc.apply(xp, gp, hp, tx, tg, th, dual)
+    y, ty = _lib.run_function(GateResidualFunc, xp, gp, hp, tx, tg, th, dual)
     return fwAD.make_dual(y, ty) if dual else y
 
 
@@ -271,14 +271,14 @@ def residual_ln_modulate(x, gate, h, shift, scale, eps: float = 1e-6):
     dt = torch.promote_types(xp.dtype, hp.dtype)
     if xp.dtype != dt:
         xp, tx = xp.to(dt), (None if tx is None else tx.to(dt))
-    y, z, ty, tz = ResidualLNModulateFunc.apply(xp, gp, hp, shp, scp, tx, tg, th, tsh, tsc, eps, _autocast_dtype(xp), dual)
+    y, z, ty, tz = _lib.run_function(ResidualLNModulateFunc, xp, gp, hp, shp, scp, tx, tg, th, tsh, tsc, eps, _autocast_dtype(xp), dual)
     return (fwAD.make_dual(y, ty), fwAD.make_dual(z, tz)) if dual else (y, z)
 
 
 def gelu_tanh(x):
     """tanh-approximated GELU."""
     (xp,), (tx,), dual = _unpack(x)
-    y, ty = GeluTanhFunc.apply(xp, tx)
+    y, ty = _lib.run_function(GeluTanhFunc, xp, tx)
     return fwAD.make_dual(y, ty) if dual else y
 
 
@@ -286,7 +286,7 @@ def silu(x):
     """``x * sigmoid(x)``; under autocast the result is produced in the autocast
     dtype (it feeds the adaLN projection, which would cast it)."""
     (xp,), (tx,), dual = _unpack(x)
-    y, ty = SiluFunc.apply(xp, tx, _autocast_dtype(xp))
+    y, ty = _lib.run_function(SiluFunc, xp, tx, _autocast_dtype(xp))
     return fwAD.make_dual(y, ty) if dual else y
 
 
@@ -295,5 +295,5 @@ def rms_norm(x, gain, eps: float = 1e-6):
     packed qkv buffer are read in place); returns a contiguous tensor.  The gain
     is treated as a constant by forward-mode AD (parameters carry no tangent)."""
     (xp,), (tx,), dual = _unpack(x)
-    y, ty = RMSNormFunc.apply(xp, gain, tx, eps, dual)
+    y, ty = _lib.run_function(RMSNormFunc, xp, gain, tx, eps, dual)
     return fwAD.make_dual(y, ty) if dual else y

@@ -103,9 +103,9 @@ def flash_attn_func(q, k, v, softmax_scale=None):
             p, tg = fwAD.unpack_dual(t)
             primals.append(p)
             tangents.append(torch.zeros_like(p) if tg is None else tg)
-        out, _, t_out = FlashAttnFunc.apply(*primals, *tangents, softmax_scale)
+        out, _, t_out = _lib.run_function(FlashAttnFunc, *primals, *tangents, softmax_scale)
         return fwAD.make_dual(out, t_out)
-    out, _, _ = FlashAttnFunc.apply(q, k, v, None, None, None, softmax_scale)
+    out, _, _ = _lib.run_function(FlashAttnFunc, q, k, v, None, None, None, softmax_scale)
     return out
 
 
@@ -163,5 +163,5 @@ def flash_attn_qkvpacked_func(qkv, softmax_scale=None):
     if qkv.dim() != 5 or qkv.shape[2] != 3:
         raise ValueError(f"expected a packed (B, L, 3, H, D) tensor, got shape {tuple(qkv.shape)}")
     p, tg = fwAD.unpack_dual(qkv)
-    out, _, t_out = FlashAttnQKVPackedFunc.apply(p, tg, softmax_scale)
+    out, _, t_out = _lib.run_function(FlashAttnQKVPackedFunc, p, tg, softmax_scale)
     return out if tg is None else fwAD.make_dual(out, t_out)
