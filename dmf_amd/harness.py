@@ -12,6 +12,7 @@ import time
 from functools import partial
 
 import torch
+import torch.autograd.forward_ad as fwAD
 
 from .dmft import DMFT_models
 
@@ -28,25 +29,34 @@ def synthetic_batch(batch: int, device, seed: int = 2, input_size: int = 32, cha
     return tuple(x.to(device) for x in (z, t, r, y, v))
 
 
-def meanflow_jvp(model, x_t, t, r, y, v):
-    """(u, du_dt) = jvp(model(., ., ., y), (x_t, t, r), (v, 1, 0)) -- loss.py:165-170."""
-    model_fn = partial(model, y=y)
-    return torch.func.jvp(model_fn, (x_t, t, r), (v, torch.ones_like(t), torch.zeros_like(r)))
+def meanflow_jvp(model, x_t, t, r, y, v, functorch: bool = True):
+    """(u, du_dt) = jvp(model(., ., ., y), (x_t, t, r), (v, 1, 0)) -- loss.py:165-170.
+
+    ``functorch=True`` is the reference's call, ``torch.func.jvp``.  ``False`` opens
+    the forward-AD dual level directly (``torch.autograd.forward_ad``), which is what
+    ``torch.func.jvp`` does underneath minus functorch's interpreter: same values,
+    but every custom autograd Function on the way costs ~20 us of host time instead
+    of ~200 us, which matters for the eagerly launched training step."""
+    if functorch:
+        return torch.func.jvp(partial(model, y=y), (x_t, t, r), (v, torch.ones_like(t), torch.zeros_like(r)))
+    with fwAD.dual_level():
+        out = model(fwAD.make_dual(x_t, v), fwAD.make_dual(t, torch.ones_like(t)), fwAD.make_dual(r, torch.zeros_like(r)), y)
+        return fwAD.unpack_dual(out)
 
 
-def meanflow_loss(model, x_t, t, r, y, v):
+def meanflow_loss(model, x_t, t, r, y, v, functorch: bool = True):
     """MeanFlow regression loss with the JVP target detached (loss.py:171-172);
     plain mean-squared error (the log-variance weighting is not part of the path)."""
-    u, du_dt = meanflow_jvp(model, x_t, t, r, y, v)
+    u, du_dt = meanflow_jvp(model, x_t, t, r, y, v, functorch)
     u_tgt = (v + (r - t) * du_dt).detach()
     return ((u - u_tgt) ** 2).mean(), u, du_dt
 
 
-def train_step(model, batch, autocast: bool = True):
+def train_step(model, batch, autocast: bool = True, functorch: bool = True):
     """Forward + JVP, then backward on the primal output only."""
     x_t, t, r, y, v = batch
     with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
-        loss, _, _ = meanflow_loss(model, x_t, t, r, y, v)
+        loss, _, _ = meanflow_loss(model, x_t, t, r, y, v, functorch)
     loss.backward()
     return loss
 
@@ -108,13 +118,15 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast, and
     (b) DMFT-XL/2 256px forward+JVP+backward, batch 32.  Variants:
     ``hip_fused_graph`` -- 'hip' attention + fused block glue, replayed as a HIP graph,
-    ``hip_fused``       -- the same, launched eagerly from Python,
+    ``hip_fused_fwad``  -- the same, launched eagerly with the forward-AD dual level opened directly,
+    ``hip_fused``       -- the same, launched eagerly through ``torch.func.jvp`` (the reference's call),
     ``hip``             -- 'hip' attention inside the reference's tensor expressions,
     ``base``            -- naive attention (the reference's own CPU-runnable operator).
     ``only`` / ``variants`` restrict the model / the variants that are run."""
     out = {}
     cases = [c for c in [("DMFT-B/2", 64, 8, False), ("DMFT-XL/2", 32, 20, True)] if only in (None, c[0])]
-    all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused", "hip", "hip", False), ("hip", "hip", "torch", False)]
+    all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused_fwad", "hip", "hip", False), ("hip_fused", "hip", "hip", False),
+                    ("hip", "hip", "torch", False)]
     if compare_base:
         all_variants.append(("base", "base", "torch", False))
     variants = [v for v in all_variants if variants is None or v[0] in variants]
@@ -123,16 +135,17 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
         data = synthetic_batch(batch, device)
         for label, op, block_ops, graphed in variants:
             model = build_model(name, op, device, dmf_depth=dmf_depth, block_ops=block_ops)
+            functorch = label != "hip_fused_fwad"
             if train:
                 def step(*batch_tensors):
                     model.zero_grad(set_to_none=True)
-                    return train_step(model, batch_tensors).detach()
+                    return train_step(model, batch_tensors, functorch=functorch).detach()
             else:
                 model.requires_grad_(False)
 
                 def step(*batch_tensors):
                     with torch.autocast("cuda", dtype=torch.bfloat16):
-                        return meanflow_jvp(model, *batch_tensors)
+                        return meanflow_jvp(model, *batch_tensors, functorch=functorch)
             run = GraphedStep(step, *data) if graphed else step
             sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
             row[f"{label}_ms_per_step"] = sec * 1e3

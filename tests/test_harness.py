@@ -156,3 +156,29 @@ def test_patch_embed_equals_strided_convolution():
     pe.fused = False
     assert torch.equal(pe(x), ref)
     assert pe.proj.weight.shape == (40, 3, 4, 4)
+
+
+def test_meanflow_jvp_direct_dual_level_equals_func_jvp():
+    m = _small("base").double()
+    z, t, r, y, v = (x.double() if x.is_floating_point() else x for x in harness.synthetic_batch(2, "cpu", input_size=8))
+    u1, du1 = harness.meanflow_jvp(m, z, t, r, y, v, functorch=True)
+    u2, du2 = harness.meanflow_jvp(m, z, t, r, y, v, functorch=False)
+    # same formulas; functorch decomposes a few ATen ops differently, so agreement is to rounding, not bitwise
+    assert torch.equal(u1, u2) and ao.rel_l2(du2, du1) < 1e-13
+
+
+@pytest.mark.gpu
+def test_fused_train_step_direct_dual_level_equals_func_jvp():
+    dev = "cuda:0"
+    m = _small("hip", block_ops="hip", input_size=32, hidden_size=288, depth=3, num_heads=4, dmf_depth=2).to(dev)
+    data = harness.synthetic_batch(4, dev)
+    grads = []
+    for functorch in (True, False):
+        m.zero_grad(set_to_none=True)
+        loss = harness.train_step(m, data, functorch=functorch)
+        grads.append((loss.detach().clone(), {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}))
+    # same kernels on both routes; the ATen ops around them may round differently under bf16 autocast
+    assert abs(float(grads[0][0]) - float(grads[1][0])) <= 1e-3 * abs(float(grads[0][0]))
+    assert grads[0][1].keys() == grads[1][1].keys()
+    worst = max(ao.rel_l2(grads[1][1][n].cpu(), grads[0][1][n].cpu()) for n in grads[0][1] if float(grads[0][1][n].abs().max()) > 0)
+    assert worst <= 2e-2, worst
