@@ -31,7 +31,7 @@ SIGNATURES = {
     "dmf_attn_bwd": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_block_workspace_floats": (c_int64, [_I] * 4),
     "dmf_ln_modulate_fwd": (c_int, [_P] * 8 + [_S] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
-    "dmf_ln_modulate_bwd": (c_int, [_P] * 7 + [_L] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
+    "dmf_ln_modulate_bwd": (c_int, [_P] * 8 + [_L] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
     "dmf_gate_residual_fwd": (c_int, [_P] * 8 + [_S] + [_I] * 3 + [_I] * 3 + [_P]),
     "dmf_gate_residual_bwd": (c_int, [_P] * 6 + [_L] + [_I] * 3 + [_I] * 3 + [_P]),
     "dmf_gelu_tanh_fwd": (c_int, [_P] * 4 + [_L, _I, _P]),
@@ -40,7 +40,6 @@ SIGNATURES = {
     "dmf_rmsnorm_bwd": (c_int, [_P] * 6 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_colsum": (c_int, [_P] * 3 + [_L, _I, _I, _I, _P]),
     "dmf_residual_ln_modulate_fwd": (c_int, [_P] * 14 + [_S] + [_I] * 3 + [_F] + [_I] * 4 + [_P]),
-    "dmf_residual_ln_modulate_bwd": (c_int, [_P] * 12 + [_L, _L] + [_I] * 3 + [_F] + [_I] * 4 + [_P]),
     "dmf_silu_fwd": (c_int, [_P] * 4 + [_L, _I, _I, _P]),
     "dmf_silu_bwd": (c_int, [_P] * 3 + [_L, _I, _I, _P]),
 }
@@ -268,10 +267,12 @@ def ln_modulate_fwd(x, shift, scale, tx=None, tshift=None, tscale=None, eps: flo
     return y, ty
 
 
-def ln_modulate_bwd(gy, x, scale, eps: float = 1e-6):
-    """(gx, gshift, gscale); gshift / gscale are dense (B, C) of scale's dtype."""
+def ln_modulate_bwd(gy, x, scale, eps: float = 1e-6, gres=None):
+    """(gx, gshift, gscale); gshift / gscale are dense (B, C) of scale's dtype.
+    ``gres`` (like x) is added to gx: the gradient x receives from elsewhere."""
     B, L, C = _blc(x)
-    gy, x = _dense(gy), _dense(x)
+    _same_dtype("ln_modulate_bwd x", x, gres)
+    gy, x, gres = _dense(gy), _dense(x), _dense(gres)
     scale, ss = _mod(scale, B, C)
     gx = _empty((B, L, C), x.dtype, x.device)
     gshift = _empty((B, C), scale.dtype, x.device)
@@ -279,8 +280,8 @@ def ln_modulate_bwd(gy, x, scale, eps: float = 1e-6):
     ws = _workspace(0, B, L, C, x.device)
     with torch.cuda.device(x.device):
         rc = load().dmf_ln_modulate_bwd(
-            gy.data_ptr(), x.data_ptr(), scale.data_ptr(), gx.data_ptr(), gshift.data_ptr(), gscale.data_ptr(), ws.data_ptr(),
-            ss, B, L, C, float(eps), _dtype_code(x), _dtype_code(scale), _dtype_code(gy), _stream(x))
+            gy.data_ptr(), x.data_ptr(), scale.data_ptr(), _ptr(gres), gx.data_ptr(), gshift.data_ptr(), gscale.data_ptr(),
+            ws.data_ptr(), ss, B, L, C, float(eps), _dtype_code(x), _dtype_code(scale), _dtype_code(gy), _stream(x))
     _check(rc, "dmf_ln_modulate_bwd")
     return gx, gshift, gscale
 
@@ -447,19 +448,9 @@ def residual_ln_modulate_fwd(x, gate, h, shift, scale, tx=None, tgate=None, th=N
 
 
 def residual_ln_modulate_bwd(gy, gz, y, h, gate, scale, eps: float = 1e-6):
-    """(gx, gh, ggate, gshift, gscale); ``gy`` may be None."""
-    B, L, C = _blc(y)
-    gy, gz, y, h = _dense(gy), _dense(gz), _dense(y), _dense(h)
-    gate, gs = _mod(gate, B, C)
-    scale, ss = _mod(scale, B, C)
-    gx = _empty((B, L, C), y.dtype, y.device)
-    gh = _empty((B, L, C), h.dtype, y.device)
-    ggate, gshift, gscale = (_empty((B, C), gate.dtype, y.device) for _ in range(3))
-    ws = _workspace(4, B, L, C, y.device)
-    with torch.cuda.device(y.device):
-        rc = load().dmf_residual_ln_modulate_bwd(
-            _ptr(gy), gz.data_ptr(), y.data_ptr(), h.data_ptr(), gate.data_ptr(), scale.data_ptr(), gx.data_ptr(), gh.data_ptr(),
-            ggate.data_ptr(), gshift.data_ptr(), gscale.data_ptr(), ws.data_ptr(), gs, ss, B, L, C, float(eps),
-            _dtype_code(y), _dtype_code(gate), _dtype_code(h), _dtype_code(gz), _stream(y))
-    _check(rc, "dmf_residual_ln_modulate_bwd")
+    """(gx, gh, ggate, gshift, gscale); ``gy`` (gradient of y from its other
+    consumers) may be None.  Two launches: the LayerNorm backward with ``gy`` folded
+    in, then the gated-residual backward on the total."""
+    gx, gshift, gscale = ln_modulate_bwd(gz, y, scale, eps, gres=gy)
+    gh, ggate = gate_residual_bwd(gx, gate, h)
     return gx, gh, ggate, gshift, gscale

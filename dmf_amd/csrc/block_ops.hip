@@ -254,7 +254,7 @@ __device__ __forceinline__ void reduce_waves_to_partial(Row<NV> (&acc)[K], float
 }
 
 struct LnBwdParams {
-  const void *gy, *x, *scale;
+  const void *gy, *x, *scale, *gres;  // gres: optional gradient reaching x from its other consumers, added to gx
   void* gx;
   float* partial;  // (B, nchunk, 2, C): [0] sum gy, [1] sum gy * xh
   int64_t ss;
@@ -294,6 +294,13 @@ __global__ __launch_bounds__(kThreads) void ln_modulate_bwd_kernel(LnBwdParams p
         g.v[j][e] *= one_plus_scale.v[j][e];
       }
     project_row(g, xh, rstd, p.C, lane);
+    if (p.gres != nullptr) {
+      load_row(p.gres, p.xbf, base, p.C, lane, xh);
+#pragma unroll
+      for (int j = 0; j < NV; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) g.v[j][e] += xh.v[j][e];
+    }
     store_row(p.gx, p.xbf, base, p.C, lane, g);
   }
   reduce_waves_to_partial<NV, 2>(acc, lds, p.partial + static_cast<int64_t>(blockIdx.x) * 2 * p.C, p.C, lane, wave);
@@ -302,7 +309,7 @@ __global__ __launch_bounds__(kThreads) void ln_modulate_bwd_kernel(LnBwdParams p
 // out[k][b][c] = sum_chunk partial[b][chunk][k][c]; out[k] dense (B, C) of the given element type.
 struct ReduceParams {
   const float* partial;
-  void* out[3];
+  void* out[2];
   int64_t total;  // B * K * C / 8 vectors
   int nchunk, K, C;
   int obf;
@@ -476,75 +483,6 @@ __global__ __launch_bounds__(kThreads) void residual_ln_modulate_fwd_kernel(ResL
       for (int e = 0; e < 8; ++e) out[e] = fmaf(t.v[j][e], 1.f + sc[e], fmaf(y.v[j][e], tsc[e], tsh[e]));
       store8(p.tz, p.zbf, base + col, out);
     }
-  }
-}
-
-struct ResLnBwdParams {
-  const void *gy, *gz, *y, *h, *gate, *scale;  // gy may be NULL (no other consumer of y)
-  void *gx, *gh;
-  float* partial;  // (B, nchunk, 3, C): [0] sum g*h (gate), [1] sum gz (shift), [2] sum gz*yh (scale)
-  int64_t gs, ss;
-  int L, C, nchunk;
-  float eps;
-  int xbf, mbf, hbf, zbf;
-};
-
-template <int NV>
-__global__ __launch_bounds__(kThreads) void residual_ln_modulate_bwd_kernel(ResLnBwdParams p) {
-  extern __shared__ float lds[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t b = blockIdx.x / p.nchunk;
-  const int chunk = blockIdx.x % p.nchunk;
-  const int r1 = min(p.L, (chunk + 1) * kChunkRows);
-  Row<NV> one_plus_scale, gate, acc[3];
-  load_row(p.scale, p.mbf, b * p.ss, p.C, lane, one_plus_scale);
-  load_row(p.gate, p.mbf, b * p.gs, p.C, lane, gate);
-#pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    zero8(acc[0].v[j]);
-    zero8(acc[1].v[j]);
-    zero8(acc[2].v[j]);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) one_plus_scale.v[j][e] += 1.f;
-  }
-  for (int r = chunk * kChunkRows + wave; r < r1; r += kWaves) {
-    const int64_t base = (b * p.L + r) * p.C;
-    Row<NV> yh, g, o;
-    load_row(p.y, p.xbf, base, p.C, lane, yh);
-    load_row(p.gz, p.zbf, base, p.C, lane, g);
-    const float rstd = normalize_row(yh, p.C, lane, p.eps);
-#pragma unroll
-    for (int j = 0; j < NV; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        acc[1].v[j][e] += g.v[j][e];
-        acc[2].v[j][e] = fmaf(g.v[j][e], yh.v[j][e], acc[2].v[j][e]);
-        g.v[j][e] *= one_plus_scale.v[j][e];
-      }
-    project_row(g, yh, rstd, p.C, lane);
-    load_row(p.gy, p.xbf, base, p.C, lane, o);   // NULL reads as zeros
-#pragma unroll
-    for (int j = 0; j < NV; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) g.v[j][e] += o.v[j][e];
-    store_row(p.gx, p.xbf, base, p.C, lane, g);
-    load_row(p.h, p.hbf, base, p.C, lane, o);
-#pragma unroll
-    for (int j = 0; j < NV; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        acc[0].v[j][e] = fmaf(g.v[j][e], o.v[j][e], acc[0].v[j][e]);
-        g.v[j][e] *= gate.v[j][e];
-      }
-    store_row(p.gh, p.hbf, base, p.C, lane, g);
-  }
-  // one accumulator at a time through the same LDS slab
-  float* out = p.partial + static_cast<int64_t>(blockIdx.x) * 3 * p.C;
-#pragma unroll
-  for (int k = 0; k < 3; ++k) {
-    Row<NV> one[1] = {acc[k]};
-    reduce_waves_to_partial<NV, 1>(one, lds, out + static_cast<int64_t>(k) * p.C, p.C, lane, wave);
-    __syncthreads();
   }
 }
 
@@ -799,12 +737,11 @@ inline int dispatch_nv(int C, F&& f) {
 }
 
 inline int reduce_partials(const float* partial, void* out0, void* out1, int B, int nchunk, int K, int C, int obf,
-                           hipStream_t s, void* out2 = nullptr) {
+                           hipStream_t s) {
   ReduceParams r{};
   r.partial = partial;
   r.out[0] = out0;
   r.out[1] = out1;
-  r.out[2] = out2;
   r.total = static_cast<int64_t>(B) * K * (C / 8);
   r.nchunk = nchunk;
   r.K = K;
@@ -847,7 +784,6 @@ int64_t dmf_block_workspace_floats(int which, int B, int L, int dim) {
     case 1: return static_cast<int64_t>(B) * nchunks(L) * dim;
     case 2: return static_cast<int64_t>(kRmsBlocksMax) * dim;
     case 3: return ((static_cast<int64_t>(B) * L + kColsumRows - 1) / kColsumRows) * dim;
-    case 4: return static_cast<int64_t>(B) * nchunks(L) * 3 * dim;
     default: return 0;
   }
 }
@@ -878,18 +814,18 @@ int dmf_ln_modulate_fwd(const void* x, const void* tx, const void* shift, const 
   });
 }
 
-int dmf_ln_modulate_bwd(const void* gy, const void* x, const void* scale, void* gx, void* gshift, void* gscale,
-                        float* workspace, int64_t scale_stride, int B, int L, int C, float eps, int x_dtype,
+int dmf_ln_modulate_bwd(const void* gy, const void* x, const void* scale, const void* gres, void* gx, void* gshift,
+                        void* gscale, float* workspace, int64_t scale_stride, int B, int L, int C, float eps, int x_dtype,
                         int mod_dtype, int gy_dtype, void* stream) {
   if (!dtype_ok(x_dtype) || !dtype_ok(mod_dtype) || !dtype_ok(gy_dtype)) return DMF_ATTN_EDTYPE;
   if (int rc = check_blc(B, L, C)) return rc;
   if (!gy || !x || !scale || !gx || !gshift || !gscale || !workspace) return DMF_ATTN_ENULL;
-  if (!aligned16(gy) || !aligned16(x) || !aligned16(gx) || !aligned16(gshift) || !aligned16(gscale) ||
-      !aligned16(workspace))
+  if (!aligned16(gy) || !aligned16(x) || !aligned16(gres) || !aligned16(gx) || !aligned16(gshift) ||
+      !aligned16(gscale) || !aligned16(workspace))
     return DMF_ATTN_EALIGN;
   if (int rc = check_mod(scale, scale_stride, mod_dtype, true)) return rc;
   LnBwdParams p{};
-  p.gy = gy; p.x = x; p.scale = scale; p.gx = gx; p.partial = workspace; p.ss = scale_stride;
+  p.gy = gy; p.x = x; p.scale = scale; p.gres = gres; p.gx = gx; p.partial = workspace; p.ss = scale_stride;
   p.L = L; p.C = C; p.nchunk = nchunks(L); p.eps = eps;
   p.xbf = x_dtype == DMF_ATTN_BF16; p.mbf = mod_dtype == DMF_ATTN_BF16; p.gbf = gy_dtype == DMF_ATTN_BF16;
   const unsigned grid = static_cast<unsigned>(B) * p.nchunk;
@@ -983,35 +919,6 @@ int dmf_residual_ln_modulate_fwd(const void* x, const void* tx, const void* gate
     if (jvp) hipLaunchKernelGGL((residual_ln_modulate_fwd_kernel<NV, true>), dim3(grid), dim3(kThreads), 0, s, p);
     else hipLaunchKernelGGL((residual_ln_modulate_fwd_kernel<NV, false>), dim3(grid), dim3(kThreads), 0, s, p);
   });
-}
-
-int dmf_residual_ln_modulate_bwd(const void* gy, const void* gz, const void* y, const void* h, const void* gate,
-                                 const void* scale, void* gx, void* gh, void* ggate, void* gshift, void* gscale,
-                                 float* workspace, int64_t gate_stride, int64_t scale_stride, int B, int L, int C,
-                                 float eps, int x_dtype, int mod_dtype, int h_dtype, int z_dtype, void* stream) {
-  if (!dtype_ok(x_dtype) || !dtype_ok(mod_dtype) || !dtype_ok(h_dtype) || !dtype_ok(z_dtype)) return DMF_ATTN_EDTYPE;
-  if (int rc = check_blc(B, L, C)) return rc;
-  if (!gz || !y || !h || !gate || !scale || !gx || !gh || !ggate || !gshift || !gscale || !workspace) return DMF_ATTN_ENULL;
-  if (!aligned16(gy) || !aligned16(gz) || !aligned16(y) || !aligned16(h) || !aligned16(gx) || !aligned16(gh) ||
-      !aligned16(ggate) || !aligned16(gshift) || !aligned16(gscale) || !aligned16(workspace))
-    return DMF_ATTN_EALIGN;
-  if (int rc = check_mod(gate, gate_stride, mod_dtype, true)) return rc;
-  if (int rc = check_mod(scale, scale_stride, mod_dtype, true)) return rc;
-  ResLnBwdParams p{};
-  p.gy = gy; p.gz = gz; p.y = y; p.h = h; p.gate = gate; p.scale = scale; p.gx = gx; p.gh = gh;
-  p.partial = workspace; p.gs = gate_stride; p.ss = scale_stride;
-  p.L = L; p.C = C; p.nchunk = nchunks(L); p.eps = eps;
-  p.xbf = x_dtype == DMF_ATTN_BF16; p.mbf = mod_dtype == DMF_ATTN_BF16;
-  p.hbf = h_dtype == DMF_ATTN_BF16; p.zbf = z_dtype == DMF_ATTN_BF16;
-  const unsigned grid = static_cast<unsigned>(B) * p.nchunk;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int rc = dispatch_nv(C, [&](auto nv) {
-    constexpr int NV = decltype(nv)::value;
-    constexpr size_t lds = (kWaves - 1) * NV * 512 * sizeof(float);
-    hipLaunchKernelGGL((residual_ln_modulate_bwd_kernel<NV>), dim3(grid), dim3(kThreads), lds, s, p);
-  });
-  if (rc) return rc;
-  return reduce_partials(workspace, ggate, gshift, B, p.nchunk, 3, C, p.mbf, s, gscale);
 }
 
 int dmf_gelu_tanh_fwd(const void* x, const void* tx, void* y, void* ty, int64_t n, int dtype, void* stream) {

@@ -41,8 +41,7 @@ extern "C" {
 
 /* Number of fp32 workspace elements a backward entry point needs.
  * `which`: 0 = dmf_ln_modulate_bwd, 1 = dmf_gate_residual_bwd (rows = B*L, dim = C),
- *          2 = dmf_rmsnorm_bwd (dim = D; B, L ignored), 3 = dmf_colsum (rows = B*L, dim = C),
- *          4 = dmf_residual_ln_modulate_bwd (rows = B*L, dim = C).
+ *          2 = dmf_rmsnorm_bwd (dim = D; B, L ignored), 3 = dmf_colsum (rows = B*L, dim = C).
  * Returns 0 on bad input. */
 DMF_ATTN_API int64_t dmf_block_workspace_floats(int which, int B, int L, int dim);
 
@@ -65,12 +64,14 @@ DMF_ATTN_API int dmf_ln_modulate_fwd(const void* x, const void* tx, const void* 
 
 /*
  * Backward of the primal of dmf_ln_modulate_fwd: given gy = dLoss/dy,
- *   gx     = rstd * (g - mean(g) - xh * mean(g * xh)),  g = gy * (1 + scale)
+ *   gx     = gres + rstd * (g - mean(g) - xh * mean(g * xh)),  g = gy * (1 + scale)
  *   gshift = sum_l gy,   gscale = sum_l gy * xh.
+ * gres (x_dtype, may be NULL = 0) is the gradient that reaches x from its other
+ * consumers (the residual path), added here instead of by a separate kernel.
  * gx: (B, L, C) of x_dtype; gshift, gscale: dense (B, C) of mod_dtype.
  */
-DMF_ATTN_API int dmf_ln_modulate_bwd(const void* gy, const void* x, const void* scale, void* gx, void* gshift,
-                                     void* gscale, float* workspace, int64_t scale_stride, int B, int L, int C,
+DMF_ATTN_API int dmf_ln_modulate_bwd(const void* gy, const void* x, const void* scale, const void* gres, void* gx,
+                                     void* gshift, void* gscale, float* workspace, int64_t scale_stride, int B, int L, int C,
                                      float eps, int x_dtype, int mod_dtype, int gy_dtype, void* stream);
 
 /*
@@ -111,18 +112,8 @@ DMF_ATTN_API int dmf_residual_ln_modulate_fwd(const void* x, const void* tx, con
                                               void* tz, const int64_t* mod_strides, int B, int L, int C, float eps,
                                               int x_dtype, int mod_dtype, int h_dtype, int z_dtype, void* stream);
 
-/*
- * Backward of the primal of dmf_residual_ln_modulate_fwd.  gy (x_dtype, may be
- * NULL) is the gradient reaching y from its other consumers, gz (z_dtype) the
- * gradient of z:  g = gy + LayerNorm-backward(gz * (1 + scale); y),
- *   gx = g (x_dtype),  gh = gate * g (h_dtype),  ggate = sum_l g * h,
- *   gshift = sum_l gz,  gscale = sum_l gz * yh   (dense (B, C) of mod_dtype).
- */
-DMF_ATTN_API int dmf_residual_ln_modulate_bwd(const void* gy, const void* gz, const void* y, const void* h,
-                                              const void* gate, const void* scale, void* gx, void* gh, void* ggate,
-                                              void* gshift, void* gscale, float* workspace, int64_t gate_stride,
-                                              int64_t scale_stride, int B, int L, int C, float eps, int x_dtype,
-                                              int mod_dtype, int h_dtype, int z_dtype, void* stream);
+/* Backward of dmf_residual_ln_modulate_fwd = dmf_ln_modulate_bwd (with the gradient of y from its other
+ * consumers passed as `gres`) followed by dmf_gate_residual_bwd on its result. */
 
 /*
  * y = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) over n elements and,

@@ -64,6 +64,10 @@ def test_ln_modulate_fwd_jvp_bwd(B, L, C, xdt, mdt, ydt):
     _close(gx, gx_ref, _tol(xdt, ydt), "gx")
     _close(gsh.view(B, 1, C), gsh_ref, _tol(mdt), "gshift")
     _close(gsc.view(B, 1, C), gsc_ref, _tol(mdt), "gscale")
+    # a gradient reaching x from elsewhere is folded into gx
+    gx2, gsh2, _ = _lib.ln_modulate_bwd(gg["gy"], gx_["x"], gm["scale"], 1e-6, gres=gx_["tx"])
+    _close(gx2, gx_ref + cx["tx"], _tol(xdt, ydt), "gx + gres")
+    assert torch.equal(gsh2, gsh)
 
 
 @pytest.mark.parametrize("B,L,C", SHAPES)
