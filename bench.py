@@ -203,6 +203,8 @@ def block_kernel_rows(device, steps=50, warmup=10):
             "ln_modulate_bwd": (lambda: _lib.ln_modulate_bwd(gyb, x, sc), n * (2 + 4 + 4)),
             "gate_residual_fwd_jvp": (lambda: _lib.gate_residual_fwd(x, gt, h, tx, tgt, th, True), n * (4 + 4 + 2 + 2 + 4 + 4)),
             "gate_residual_bwd": (lambda: _lib.gate_residual_bwd(gyf, gt, h), n * (4 + 2 + 2)),
+            "residual_ln_modulate_fwd_jvp": (lambda: _lib.residual_ln_modulate_fwd(x, gt, h, sh, sc, tx, tgt, th, tsh, tsc, 1e-6, bf16, True),
+                                             n * (4 + 4 + 2 + 2 + 4 + 4 + 2 + 2)),
             "gelu_tanh_fwd_jvp": (lambda: _lib.gelu_tanh_fwd(u, tu), 4 * n * 2 * 4),
             "gelu_tanh_bwd": (lambda: _lib.gelu_tanh_bwd(tu, u), 4 * n * 2 * 3),
             "colsum_4C": (lambda: _lib.colsum(u.view(B * L, 4 * C), f32), 4 * n * 2),
