@@ -220,7 +220,11 @@ class DualLinearFunc(torch.autograd.Function):
         gx = (g2 @ w).reshape(x.shape).to(x.dtype) if ctx.needs_input_grad[0] else None
         gw = None
         if ctx.needs_input_grad[2]:
-            gw = (g2.t() @ x.reshape(-1, x.shape[-1]).to(w.dtype)).to(ctx.weight_dtype)
+            x2 = x.reshape(-1, x.shape[-1]).to(w.dtype)
+            if g2.is_cuda and g2.dtype != ctx.weight_dtype and ctx.weight_dtype == torch.float32:
+                gw = torch.mm(g2.t(), x2, out_dtype=torch.float32)   # the GEMM stores its fp32 accumulators: no cast kernel
+            else:
+                gw = (g2.t() @ x2).to(ctx.weight_dtype)
         gb = None
         if ctx.bias_dtype is not None and ctx.needs_input_grad[3]:
             # torch's multi-block column reduction clears its scratch with a memset node, which does not survive
