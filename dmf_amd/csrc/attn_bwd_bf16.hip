@@ -44,13 +44,15 @@ __device__ __forceinline__ void zero_pads(char* smem, int tile_off, int tid) {
 }
 
 // ------------------------------------------------------------------ dQ kernel
-template <int D>
+// SUB = 32-key tiles per stage (and per work-group barrier).
+template <int D, int SUB>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParams p) {
   using F = BwdFastCfg<D>;
   using T = __bf16;
   constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR;
   constexpr bool TAIL = F::TAIL;
-  constexpr int STAGE = 2 * F::TBYTES;   // K | V
+  constexpr int PAIR = 2 * F::TBYTES;    // one 32-key tile: K | V
+  constexpr int STAGE = SUB * PAIR;
   constexpr int V_OFF = F::TBYTES;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -64,8 +66,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
   const int q0 = qb * 128;
   auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
 
-  zero_pads<STAGE, P - VPR, P, VPR>(smem, 0, tid);
-  zero_pads<STAGE, P - VPR, P, VPR>(smem, V_OFF, tid);
+#pragma unroll
+  for (int sub = 0; sub < SUB; ++sub) {
+    zero_pads<STAGE, P - VPR, P, VPR>(smem, sub * PAIR, tid);
+    zero_pads<STAGE, P - VPR, P, VPR>(smem, sub * PAIR + V_OFF, tid);
+  }
 
   // ---- this lane's query row: Q (times scale*log2e), dout, delta, lse
   const int qrow = q0 + wave * 32 + c32;
@@ -103,23 +108,33 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
   const uint32_t rb_k = (uint32_t)p.st[2][1] * 2, rb_v = (uint32_t)p.st[3][1] * 2;
   const __amdgpu_buffer_rsrc_t rs_k = make_rows_rsrc(reinterpret_cast<const T*>(p.k) + base(2), rb_k, p.Lkv, D * 2);
   const __amdgpu_buffer_rsrc_t rs_v = make_rows_rsrc(reinterpret_cast<const T*>(p.v) + base(3), rb_v, p.Lkv, D * 2);
-  auto issue = [&](int it) {
-    char* st = smem + (it & 1) * STAGE;
-    issue_tile_rows<P, VPR>(rs_k, rb_k, (uint32_t)it * 32 * rb_k, st, wave, lane);
-    issue_tile_rows<P, VPR>(rs_v, rb_v, (uint32_t)it * 32 * rb_v, st + V_OFF, wave, lane);
+  const int ntiles = (p.Lkv + 31) / 32;             // 32-key tiles
+  const int nstages = (ntiles + SUB - 1) / SUB;
+  auto issue = [&](int is) {
+    char* st = smem + (is & 1) * STAGE;
+#pragma unroll
+    for (int sub = 0; sub < SUB; ++sub) {
+      const int it = is * SUB + sub;
+      if (it < ntiles) {   // wave-uniform
+        issue_tile_rows<P, VPR>(rs_k, rb_k, (uint32_t)it * 32 * rb_k, st + sub * PAIR, wave, lane);
+        issue_tile_rows<P, VPR>(rs_v, rb_v, (uint32_t)it * 32 * rb_v, st + sub * PAIR + V_OFF, wave, lane);
+      }
+    }
   };
   const uint32_t row_addr = lds_addr(smem) + c32 * STR * 2 + g * 16;
   const uint32_t col_addr = lds_addr(smem) + ((4 * g + ((lane & 15) >> 2)) * STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
   const uint32_t tail_addr = lds_addr(smem) + tail_lane_offset(lane, STR, 32 * NMT) * 2;
 
-  const int ntiles = (p.Lkv + 31) / 32;
   issue(0);
-  for (int it = 0; it < ntiles; ++it) {
+  for (int is = 0; is < nstages; ++is) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     lds_barrier();
-    if (it + 1 < ntiles) issue(it + 1);
-    const uint32_t ra = row_addr + (it & 1) * STAGE, ca = col_addr + (it & 1) * STAGE;
+    if (is + 1 < nstages) issue(is + 1);
+   for (int sub = 0; sub < SUB; ++sub) {
+    const int it = is * SUB + sub;
+    if (it >= ntiles) break;             // wave-uniform
+    const uint32_t ra = row_addr + (is & 1) * STAGE + sub * PAIR, ca = col_addr + (is & 1) * STAGE + sub * PAIR;
 
     // ---- S^T = K Q^T (log2 units), dP^T = V dout^T
     f32x16 S = {0}, dP = {0};
@@ -159,7 +174,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
         constexpr int gi = decltype(gc)::value;
         constexpr bool more = gi + 1 < NGT;
         if constexpr (gi + 1 < NG) kk[(gi + 1) & 1] = lds_tr16_issue<lo_off(gi + 1), lo_off(gi + 1) + 8 * STR * 2>(ca);
-        else if constexpr (more) kk[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(tail_addr + (it & 1) * STAGE);
+        else if constexpr (more) kk[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(tail_addr + (is & 1) * STAGE + sub * PAIR);
         lds_tr16_wait<more ? 2 : 0>(kk[gi & 1]);
         if constexpr (gi < NG) {
           mma_col<T>(dQ[gi % NMT], tr_operand(kk[gi & 1]), ds[gi / NMT]);
@@ -171,6 +186,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
         }
       });
     }
+   }
   }
   store_rows_transposed<T, D, 4, NMT>(reinterpret_cast<T*>(smem), reinterpret_cast<T*>(p.dq) + base(5), p.st[5][1], q0, p.Lq, tid,
                                       [&](int t, int i) { return dQ[t][i] * p.scale; },
@@ -337,12 +353,15 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
   constexpr int tiles = 2 * (2 * F::TBYTES + F::STAT) + 512;
   constexpr int stage = 128 * Cfg<__bf16, D>::OROWV * 16;
   constexpr int smem = tiles > stage ? tiles : stage;
-  auto k1 = attn_bwd_dq_bf16_kernel<D>;
+  constexpr int kDqSub = 2;   // two 32-key tiles per barrier in the dQ kernel (+3 % over one; four would leave one work-group per CU)
+  constexpr int tiles1 = 2 * kDqSub * 2 * F::TBYTES + 512;
+  constexpr int smem1 = tiles1 > stage ? tiles1 : stage;
+  auto k1 = attn_bwd_dq_bf16_kernel<D, kDqSub>;
   auto k2 = attn_bwd_dkv_bf16_kernel<D>;
   static bool lds_ok1[64] = {}, lds_ok2[64] = {};
-  if (!ensure_dynamic_lds(k1, smem, lds_ok1) || !ensure_dynamic_lds(k2, smem, lds_ok2)) return -7;
+  if (!ensure_dynamic_lds(k1, smem1, lds_ok1) || !ensure_dynamic_lds(k2, smem, lds_ok2)) return -7;
   const uint32_t nqb = (p.Lq + 127) / 128, nkb = (p.Lkv + 127) / 128;
-  hipLaunchKernelGGL(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
+  hipLaunchKernelGGL(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem1, stream, p);
   if (hipGetLastError() != hipSuccess) return -7;
   hipLaunchKernelGGL(k2, dim3(nkb * (uint32_t)BH), dim3(256), smem, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : -7;
