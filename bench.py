@@ -180,6 +180,21 @@ def device_probes():
     return out
 
 
+def per_launch_stats(fn, iters=50):
+    """Median and minimum duration (ms) of single launches, one HIP event pair per launch."""
+    import torch
+
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    torch.cuda.synchronize()
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in ev)
+    return ts[len(ts) // 2], ts[0]
+
+
 def block_kernel_rows(device, steps=50, warmup=10):
     """HBM-bound block-glue kernels at the two end-to-end shapes: algorithmic
     bytes (each operand read once, each result written once) / launch time."""
@@ -266,6 +281,7 @@ def main():
     ms, wall_ms = time_gpu(lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale), args.steps, args.warmup)
     flops = attn_flops(B, H, N, D, "fwd_jvp")
     tflops = flops / (ms * 1e-3) / 1e12
+    ms_median, ms_min = per_launch_stats(lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale))
     result = {
         "metric": "attn_fwd_jvp_tflops", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
@@ -273,7 +289,7 @@ def main():
         "config": {"workload": f"{name}: attention fwd+JVP B={B} H={H} N={N} D={D} bf16"
                                + (" q,k RMS-normalised" if WORKLOADS[name][4] else ""),
                    "flops_per_step": flops, "hbm_bytes_per_step": attn_bytes(B, H, N, D, "fwd_jvp"),
-                   "wall_ms_per_step": wall_ms},
+                   "wall_ms_per_step": wall_ms, "single_launch_ms_median": ms_median, "single_launch_ms_min": ms_min},
         "roofline": roofline(name, ms),
     }
 
