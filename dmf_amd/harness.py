@@ -115,8 +115,10 @@ def _time(fn, steps: int, warmup: int = 2) -> float:
 
 
 def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=None, variants=None) -> dict:
-    """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast, and
-    (b) DMFT-XL/2 256px forward+JVP+backward, batch 32.  Variants:
+    """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast,
+    (b) DMFT-XL/2 256px forward+JVP+backward, batch 32, and (c) DMFT-B/2 primal-only
+    no-grad forward at batch 128 -- the call mode of the guidance branch
+    (loss.py:64-69, a 2B batch) and of a sampler step (samplers.py:69-100).  Variants:
     ``hip_fused_graph`` -- 'hip' attention + fused block glue, replayed as a HIP graph,
     ``hip_fused_fwad``  -- the same, launched eagerly with the forward-AD dual level opened directly,
     ``hip_fused``       -- the same, launched eagerly through ``torch.func.jvp`` (the reference's call),
@@ -124,33 +126,44 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     ``base``            -- naive attention (the reference's own CPU-runnable operator).
     ``only`` / ``variants`` restrict the model / the variants that are run."""
     out = {}
-    cases = [c for c in [("DMFT-B/2", 64, 8, False), ("DMFT-XL/2", 32, 20, True)] if only in (None, c[0])]
+    all_cases = [("DMFT-B/2", "DMFT-B/2", 64, 8, "jvp"), ("DMFT-XL/2", "DMFT-XL/2", 32, 20, "train"),
+                 ("DMFT-B/2 no-grad", "DMFT-B/2", 128, 8, "nograd")]
+    cases = [c for c in all_cases if only in (None, c[0])]
     all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused_fwad", "hip", "hip", False), ("hip_fused", "hip", "hip", False),
                     ("hip", "hip", "torch", False)]
     if compare_base:
         all_variants.append(("base", "base", "torch", False))
     variants = [v for v in all_variants if variants is None or v[0] in variants]
-    for name, batch, dmf_depth, train in cases:
-        row = {"batch": batch, "mode": "fwd+jvp+bwd" if train else "fwd+jvp", "dtype": "bf16 autocast"}
+    modes = {"jvp": "fwd+jvp", "train": "fwd+jvp+bwd", "nograd": "primal-only forward, no grad (guidance / sampler call)"}
+    for key, name, batch, dmf_depth, mode in cases:
+        row = {"batch": batch, "mode": modes[mode], "dtype": "bf16 autocast"}
         data = synthetic_batch(batch, device)
         for label, op, block_ops, graphed in variants:
+            if mode == "nograd" and label == "hip_fused_fwad":
+                continue   # no JVP in this mode
             model = build_model(name, op, device, dmf_depth=dmf_depth, block_ops=block_ops)
             functorch = label != "hip_fused_fwad"
-            if train:
+            if mode == "train":
                 def step(*batch_tensors):
                     model.zero_grad(set_to_none=True)
                     return train_step(model, batch_tensors, functorch=functorch).detach()
-            else:
+            elif mode == "jvp":
                 model.requires_grad_(False)
 
                 def step(*batch_tensors):
                     with torch.autocast("cuda", dtype=torch.bfloat16):
                         return meanflow_jvp(model, *batch_tensors, functorch=functorch)
+            else:
+                model.requires_grad_(False)
+
+                def step(z, t, r, y, v):
+                    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                        return model(z, t, r, y)
             run = GraphedStep(step, *data) if graphed else step
             sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
             row[f"{label}_ms_per_step"] = sec * 1e3
             row[f"{label}_images_per_s"] = batch / sec
             del model, run, step
             torch.cuda.empty_cache()
-        out[name] = row
+        out[key] = row
     return out
