@@ -118,7 +118,9 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast,
     (b) DMFT-XL/2 256px forward+JVP+backward, batch 32, and (c) DMFT-B/2 primal-only
     no-grad forward at batch 128 -- the call mode of the guidance branch
-    (loss.py:64-69, a 2B batch) and of a sampler step (samplers.py:69-100).  Variants:
+    (loss.py:64-69, a 2B batch) and of a sampler step (samplers.py:69-100) -- and
+    (d) DMFT-XL/2 at 512px (1024 tokens) with qk-norm, forward+JVP, batch 16: the
+    caller of the headline attention shape.  Variants:
     ``hip_fused_graph`` -- 'hip' attention + fused block glue, replayed as a HIP graph,
     ``hip_fused_fwad``  -- the same, launched eagerly with the forward-AD dual level opened directly,
     ``hip_fused``       -- the same, launched eagerly through ``torch.func.jvp`` (the reference's call),
@@ -126,8 +128,10 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     ``base``            -- naive attention (the reference's own CPU-runnable operator).
     ``only`` / ``variants`` restrict the model / the variants that are run."""
     out = {}
-    all_cases = [("DMFT-B/2", "DMFT-B/2", 64, 8, "jvp"), ("DMFT-XL/2", "DMFT-XL/2", 32, 20, "train"),
-                 ("DMFT-B/2 no-grad", "DMFT-B/2", 128, 8, "nograd")]
+    # (key, model, batch, dmf_depth, mode, latent size, qk_norm)
+    all_cases = [("DMFT-B/2", "DMFT-B/2", 64, 8, "jvp", 32, False), ("DMFT-XL/2", "DMFT-XL/2", 32, 20, "train", 32, False),
+                 ("DMFT-B/2 no-grad", "DMFT-B/2", 128, 8, "nograd", 32, False),
+                 ("DMFT-XL/2 512px qk-norm", "DMFT-XL/2", 16, 20, "jvp", 64, True)]
     cases = [c for c in all_cases if only in (None, c[0])]
     all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused_fwad", "hip", "hip", False), ("hip_fused", "hip", "hip", False),
                     ("hip", "hip", "torch", False)]
@@ -135,13 +139,13 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
         all_variants.append(("base", "base", "torch", False))
     variants = [v for v in all_variants if variants is None or v[0] in variants]
     modes = {"jvp": "fwd+jvp", "train": "fwd+jvp+bwd", "nograd": "primal-only forward, no grad (guidance / sampler call)"}
-    for key, name, batch, dmf_depth, mode in cases:
-        row = {"batch": batch, "mode": modes[mode], "dtype": "bf16 autocast"}
-        data = synthetic_batch(batch, device)
+    for key, name, batch, dmf_depth, mode, input_size, qk_norm in cases:
+        row = {"batch": batch, "mode": modes[mode], "dtype": "bf16 autocast", "tokens": (input_size // 2) ** 2, "qk_norm": qk_norm}
+        data = synthetic_batch(batch, device, input_size=input_size)
         for label, op, block_ops, graphed in variants:
             if mode == "nograd" and label == "hip_fused_fwad":
                 continue   # no JVP in this mode
-            model = build_model(name, op, device, dmf_depth=dmf_depth, block_ops=block_ops)
+            model = build_model(name, op, device, qk_norm=qk_norm, input_size=input_size, dmf_depth=dmf_depth, block_ops=block_ops)
             functorch = label != "hip_fused_fwad"
             if mode == "train":
                 def step(*batch_tensors):
