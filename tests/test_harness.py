@@ -208,3 +208,24 @@ def test_dmft_b2_full_architecture_fused_graph_vs_base():
         u, du = graphed(*data)
         assert ao.rel_l2(u.float().cpu(), u_ref.float().cpu()) <= 3e-2
         assert ao.rel_l2(du.float().cpu(), du_ref.float().cpu()) <= 3e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,qk_norm", [("DMFT-S/2", False), ("DMFT-B/4", True), ("DMFT-L/8", False), ("DMFT-M/4", True)])
+def test_registry_models_fused_vs_base(name, qk_norm):
+    """Other sizes of the reference's registry (models/dmft.py:154-175): head dim 64, hidden 384 / 768 / 1024,
+    64 and 16 tokens (patch 4 and 8): forward+JVP and gradients, fused path vs the reference expressions, fp32."""
+    dev = "cuda:0"
+    m_ref = harness.build_model(name, "base", dev, qk_norm=qk_norm, dmf_depth=2)
+    m = harness.build_model(name, "hip", dev, qk_norm=qk_norm, dmf_depth=2, block_ops="hip")
+    m.load_state_dict(m_ref.state_dict())
+    data = harness.synthetic_batch(2, dev)
+    outs = []
+    for mod in (m, m_ref):
+        loss, u, du = harness.meanflow_loss(mod, *data)
+        loss.backward()
+        outs.append((u.detach().cpu(), du.detach().cpu()))
+    assert ao.rel_l2(outs[0][0], outs[1][0]) <= 2e-4 and ao.rel_l2(outs[0][1], outs[1][1]) <= 2e-4
+    worst = max(ao.rel_l2(p.grad.cpu(), q.grad.cpu()) for (n, p), (_, q) in zip(m.named_parameters(), m_ref.named_parameters())
+                if q.grad is not None and float(q.grad.abs().max()) > 0)
+    assert worst <= 1e-3, worst
