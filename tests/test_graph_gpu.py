@@ -1,18 +1,27 @@
 """HIP-graph replay of the fused MeanFlow step (dmf_amd.harness.GraphedStep).
 
-A captured graph must give, on every replay, exactly what the eager step gives
-on the same inputs -- with unrelated eager work and host synchronisation between
+A captured graph must give, on every replay, what the eager step gives on the
+same inputs -- with unrelated eager work and host synchronisation between
 replays, and with inputs that change from replay to replay.  (A reduction that
 clears scratch memory through a memset node passes the first replay and fails
-later ones; this is the test that catches it.)"""
+later ones, by factors of 1 to 1000 relative; this is the test that catches it.)
+The kernels are the same on both routes, so results normally agree bit for bit;
+the assertions allow rounding-level differences (a library GEMM may pick a
+different accumulation order from one launch to the next) and nothing more."""
 import pytest
 import torch
 
 from dmf_amd import harness
 from dmf_amd.dmft import DMFT
+from oracle import attn_oracle as ao
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+TOL = 2e-3   # relative L2; bf16 rounding of one GEMM output is ~4e-3 per element
+
+
+def _same(a, b):
+    return torch.equal(a, b) or ao.rel_l2(a.float().cpu(), b.float().cpu()) <= TOL
 
 
 def _model(**kw):
@@ -41,7 +50,7 @@ def test_graphed_jvp_step_replays_match_eager():
         for b, (u_ref, du_ref) in zip(batches, eager):
             u, du = step(*b)
             torch.cuda.synchronize()
-            assert torch.equal(u, u_ref) and torch.equal(du, du_ref), f"replay {rep} differs from eager"
+            assert _same(u, u_ref) and _same(du, du_ref), f"replay {rep} differs from eager"
             _eager_noise()
 
 
@@ -67,7 +76,7 @@ def test_graphed_train_step_replays_match_eager():
         for b, (loss_ref, grads_ref) in zip(batches, eager):
             loss = step(*b)
             torch.cuda.synchronize()
-            assert torch.equal(loss, loss_ref)
-            bad = [n for n, g in grads_ref.items() if not torch.equal(params[n].grad, g)]
+            assert _same(loss, loss_ref)
+            bad = [n for n, g in grads_ref.items() if not _same(params[n].grad, g)]
             assert not bad, f"replay {rep}: gradients differ from eager for {bad[:6]}"
             _eager_noise()
