@@ -13,5 +13,6 @@ All device work is done by hand-written gfx950 kernels reached through the
 C ABI in ``include/dmf_attn.h`` (``dmf_amd/libdmf_attn.so``); there is no
 fallback path: if the library is missing, calls raise.
 """
-from .flash_attention_hip_jvp import FlashAttnFunc, FlashAttnQKVPackedFunc, flash_attn_func, flash_attn_qkvpacked_func  # noqa: F401
+from .flash_attention_hip_jvp import (FlashAttnFunc, FlashAttnQKVPackedFunc, QKNormAttnQKVPackedFunc, flash_attn_func,  # noqa: F401
+                                      flash_attn_qknorm_qkvpacked_func, flash_attn_qkvpacked_func)
 from .layers import attn_op, ATTN_FUNCS  # noqa: F401

@@ -363,17 +363,25 @@ def rmsnorm_fwd(x, gain, tx=None, eps: float = 1e-6, jvp=False):
     return y, ty
 
 
-def rmsnorm_bwd(gy, x, gain, eps: float = 1e-6):
-    """(gx, ggain): gx contiguous (B, L, H, D), ggain (D) of gain's dtype."""
+def rmsnorm_bwd(gy, x, gain, eps: float = 1e-6, out=None):
+    """(gx, ggain): gx a fresh contiguous (B, L, H, D) tensor -- or ``out``, any
+    (B, L, H, D) view with unit last-dim stride and 16-byte aligned rows (e.g. one
+    slot of a packed qkv gradient buffer), filled in place; ggain (D) of gain's dtype."""
     _check_inputs(x, gy)
     x, gy, gain = _prep(x), _dense(gy), _dense(gain)
     B, L, H, D = x.shape
-    gx = _empty((B, L, H, D), x.dtype, x.device)
+    if out is None:
+        gx = _empty((B, L, H, D), x.dtype, x.device)
+    else:
+        gx = _raw(out)
+        _check_inputs(x, gx)
+        if gx.shape != x.shape:
+            raise ValueError("rmsnorm_bwd: `out` must have the shape of x")
     ggain = _empty((D,), gain.dtype, x.device)
     ws = _workspace(2, B, L, D, x.device)
     with torch.cuda.device(x.device):
         rc = load().dmf_rmsnorm_bwd(
-            gy.data_ptr(), x.data_ptr(), gain.data_ptr(), gx.data_ptr(), ggain.data_ptr(), ws.data_ptr(), _strides(x),
+            gy.data_ptr(), x.data_ptr(), gain.data_ptr(), gx.data_ptr(), ggain.data_ptr(), ws.data_ptr(), _strides(x, gx),
             B, L, H, D, float(eps), _dtype_code(x), _dtype_code(gain), _stream(x))
     _check(rc, "dmf_rmsnorm_bwd")
     return gx, ggain

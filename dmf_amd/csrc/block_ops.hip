@@ -539,7 +539,7 @@ struct RmsParams {
   const void *x, *tx, *gain, *gy;
   void *y, *ty;    // backward: y = gx
   float* partial;  // backward: (nblocks, D)
-  int64_t rows, sx[3], stx[3];
+  int64_t rows, sx[3], stx[3];   // element strides {sB, sL, sH} of x and of tx (forward) / gx (backward)
   int L, H, D;
   float eps;
   int bf, gbf;
@@ -623,7 +623,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(RmsParams p) {
         acc[e] = fmaf(g[e], x[e] * r, acc[e]);
         out[e] = fmaf(g[e] * gain[e], r, -x[e] * c);
       }
-      store8(p.y, p.bf, row * p.D + col, out);
+      store8(p.y, p.bf, strided_row(row, p.L, p.H, p.stx) + col, out);   // stx: strides of gx in this kernel
     }
   }
   // the four lane groups of a wave, then the waves of the work-group
@@ -1001,10 +1001,10 @@ int dmf_rmsnorm_bwd(const void* gy, const void* x, const void* gain, void* gx, v
                     void* stream) {
   if (int rc = check_rms(B, L, H, D, dtype, gain_dtype)) return rc;
   if (!gy || !x || !gain || !gx || !ggain || !workspace || !strides) return DMF_ATTN_ENULL;
-  if (!aligned16(gy) || !aligned16(gain) || !aligned16(gx) || !aligned16(ggain) || !aligned16(workspace))
-    return DMF_ATTN_EALIGN;
+  if (!aligned16(gy) || !aligned16(gain) || !aligned16(ggain) || !aligned16(workspace)) return DMF_ATTN_EALIGN;
   RmsParams p{};
   if (int rc = check_blhd(x, strides, ebytes(dtype), p.sx)) return rc;
+  if (int rc = check_blhd(gx, strides + 4, ebytes(dtype), p.stx)) return rc;
   p.x = x; p.gy = gy; p.gain = gain; p.y = gx; p.partial = workspace;
   p.rows = static_cast<int64_t>(B) * L * H;
   p.L = L; p.H = H; p.D = D; p.eps = eps;

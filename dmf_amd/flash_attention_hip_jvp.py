@@ -165,3 +165,63 @@ def flash_attn_qkvpacked_func(qkv, softmax_scale=None):
     p, tg = fwAD.unpack_dual(qkv)
     out, _, t_out = _lib.run_function(FlashAttnQKVPackedFunc, p, tg, softmax_scale)
     return out if tg is None else fwAD.make_dual(out, t_out)
+
+
+class QKNormAttnQKVPackedFunc(torch.autograd.Function):
+    """(qkv, tqkv, q_gain, k_gain, eps, softmax_scale) -> (o, lse, to): per-head RMS
+    norm of the q and k slots of a packed (B, L, 3, H, D) projection output followed
+    by attention -- ``q, k = self.q_norm(q), self.k_norm(k); x = self.attn(q, k, v)``
+    (reference models/layers.py:147-151) -- as one autograd node.  Forward is the
+    fused RMS-norm kernel (primal + tangent) on each slot, read in place, then the
+    attention kernel; backward sends dv and the two norm gradients straight into the
+    three slots of one packed gradient buffer."""
+
+    @staticmethod
+    def forward(qkv, tqkv, q_gain, k_gain, eps, softmax_scale):
+        q, k, v = qkv.unbind(2)
+        scale = _default_scale(q, softmax_scale)
+        jvp = tqkv is not None
+        tq, tk, tv = tqkv.unbind(2) if jvp else (None, None, None)
+        qn, tqn = _lib.rmsnorm_fwd(q, q_gain, tq, eps, jvp)
+        kn, tkn = _lib.rmsnorm_fwd(k, k_gain, tk, eps, jvp)
+        if jvp:
+            o, to, lse = _lib.fwd_jvp(qn, kn, v, tqn, tkn, tv, scale)
+        else:
+            o, lse = _lib.fwd(qn, kn, v, scale, need_lse=True)
+            to = None
+        return o, lse, to, qn, kn
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        qkv, _, q_gain, k_gain, eps, softmax_scale = inputs
+        o, lse, _, qn, kn = outputs
+        ctx.save_for_backward(qkv, q_gain, k_gain, qn, kn, o, lse)
+        ctx.mark_non_differentiable(qn, kn)
+        ctx.eps, ctx.softmax_scale = eps, _default_scale(qkv, softmax_scale)
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, dout, *ignored):
+        if dout is None:
+            return (None,) * 6
+        qkv, q_gain, k_gain, qn, kn, o, lse = ctx.saved_tensors
+        q, k, v = qkv.unbind(2)
+        gqkv = torch.empty(qkv.shape, dtype=qkv.dtype, device=qkv.device)
+        gq, gk, gv = gqkv.unbind(2)
+        dqn = torch.empty(qn.shape, dtype=qn.dtype, device=qn.device)
+        dkn = torch.empty(kn.shape, dtype=kn.dtype, device=kn.device)
+        _lib.bwd(dout, qn, kn, v, o, lse, ctx.softmax_scale, out=(dqn, dkn, gv))
+        _, gq_gain = _lib.rmsnorm_bwd(dqn, q, q_gain, ctx.eps, out=gq)
+        _, gk_gain = _lib.rmsnorm_bwd(dkn, k, k_gain, ctx.eps, out=gk)
+        return gqkv, None, gq_gain, gk_gain, None, None
+
+
+def flash_attn_qknorm_qkvpacked_func(qkv, q_gain, k_gain, eps: float = 1e-6, softmax_scale=None):
+    """RMS-normalise the q and k slots of a packed (B, L, 3, H, D) tensor per head
+    (gains ``q_gain``, ``k_gain`` of shape (D)) and attend; returns (B, L, H, D).
+    Dual in -> dual out; the gains are constants of the tangent map."""
+    if qkv.dim() != 5 or qkv.shape[2] != 3:
+        raise ValueError(f"expected a packed (B, L, 3, H, D) tensor, got shape {tuple(qkv.shape)}")
+    p, tg = fwAD.unpack_dual(qkv)
+    out, _, t_out, _, _ = _lib.run_function(QKNormAttnQKVPackedFunc, p, tg, q_gain, k_gain, eps, softmax_scale)
+    return out if tg is None else fwAD.make_dual(out, t_out)

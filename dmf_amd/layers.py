@@ -17,6 +17,7 @@ from torch import Tensor
 
 from . import block_ops as fused
 from .flash_attention_hip_jvp import flash_attn_func as hip_func
+from .flash_attention_hip_jvp import flash_attn_qknorm_qkvpacked_func as hip_qknorm_qkvpacked_func
 from .flash_attention_hip_jvp import flash_attn_qkvpacked_func as hip_qkvpacked_func
 
 # values accepted by --attn-func; "hip" is the one this package adds
@@ -156,13 +157,18 @@ class Attention(nn.Module):
         self.k_norm = RMSNorm(self.head_dim, block_ops=block_ops) if qk_norm else nn.Identity()
         self.proj = Linear(dim, dim, bias=proj_bias, block_ops=block_ops)
         self.attn = partial(attn_op, op=attn_func)
-        # without qk-norm the 'hip' operator can take the projection output as it is
-        self.packed = _check_block_ops(block_ops) and attn_func == "hip" and not qk_norm
+        # the 'hip' operator can take the projection output as it is (with or without qk-norm)
+        self.packed = _check_block_ops(block_ops) and attn_func == "hip"
+        self.qk_norm = qk_norm
 
     def forward(self, x: Tensor) -> Tensor:
         B, L, C = x.shape
         if self.packed:
-            x = hip_qkvpacked_func(self.qkv(x).reshape(B, L, 3, self.num_heads, self.head_dim))
+            qkv = self.qkv(x).reshape(B, L, 3, self.num_heads, self.head_dim)
+            if self.qk_norm:
+                x = hip_qknorm_qkvpacked_func(qkv, self.q_norm.scale, self.k_norm.scale, self.q_norm.eps)
+            else:
+                x = hip_qkvpacked_func(qkv)
             return self.proj(x.reshape(B, L, C))
         qkv = self.qkv(x).reshape(B, L, 3, self.num_heads, self.head_dim).permute(2, 0, 1, 3, 4)
         q, k, v = qkv.unbind(0)  # each (B, L, H, D), strides (3LHD, 3HD, D, 1)

@@ -156,8 +156,9 @@ DMF_ATTN_API int dmf_rmsnorm_fwd(const void* x, const void* tx, const void* gain
 /*
  * Backward of the primal of dmf_rmsnorm_fwd:
  *   g = gy * gain,  gx = r * g - x * r^3 * mean(x * g),  ggain = sum_rows gy * x * r.
- * x: strided as above (strides = {x[4]}); gy, gx: dense (B, L, H, D); ggain: (D)
- * of gain_dtype.
+ * x and gx: strided as above (strides = {x[4], gx[4]}; gx may be one slot of a
+ * packed (B, L, 3, H, D) gradient buffer); gy: dense (B, L, H, D); ggain: (D) of
+ * gain_dtype.
  */
 DMF_ATTN_API int dmf_rmsnorm_bwd(const void* gy, const void* x, const void* gain, void* gx, void* ggain,
                                  float* workspace, const int64_t* strides, int B, int L, int H, int D, float eps,

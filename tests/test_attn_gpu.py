@@ -263,3 +263,41 @@ def test_qkvpacked_func_matches_unpacked_and_writes_packed_grads(dtype):
     assert torch.equal(o3, o1.detach()) and torch.equal(to3, to1.detach())
     with pytest.raises(ValueError):
         dmf_amd.flash_attn_qkvpacked_func(qkv[:, :, 0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_qknorm_qkvpacked_func_matches_composition(dtype):
+    """RMS-norm of the q / k slots + attention as one node on the packed buffer: same
+    kernels as rms_norm -> rms_norm -> flash_attn_func on the slices, so the same bits
+    for outputs, tangents and the packed gradient (which the kernels fill in place)."""
+    import dmf_amd
+    from dmf_amd import block_ops
+    B, L, H, D = 2, 136, 3, 72
+    g = torch.Generator().manual_seed(23)
+    qkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(DEV)
+    tqkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(DEV)
+    dout = torch.randn(B, L, H, D, generator=g).to(dtype).to(DEV)
+    gq = (1 + 0.2 * torch.randn(D, generator=g)).to(DEV).requires_grad_()
+    gk = (1 + 0.2 * torch.randn(D, generator=g)).to(DEV).requires_grad_()
+    gq2, gk2 = gq.detach().clone().requires_grad_(), gk.detach().clone().requires_grad_()
+    a = qkv.clone().requires_grad_()
+    b = qkv.clone().requires_grad_()
+
+    def composed(x):
+        q, k, v = x.unbind(2)
+        return dmf_amd.flash_attn_func(block_ops.rms_norm(q, gq2), block_ops.rms_norm(k, gk2), v)
+
+    o1, to1 = torch.func.jvp(lambda x: dmf_amd.flash_attn_qknorm_qkvpacked_func(x, gq, gk), (a,), (tqkv,))
+    o2, to2 = torch.func.jvp(composed, (b,), (tqkv,))
+    assert torch.equal(o1, o2) and torch.equal(to1, to2)
+    o1.backward(dout)
+    o2.backward(dout)
+    assert torch.equal(a.grad, b.grad)
+    assert torch.equal(gq.grad, gq2.grad) and torch.equal(gk.grad, gk2.grad)
+    with torch.no_grad():
+        assert torch.equal(dmf_amd.flash_attn_qknorm_qkvpacked_func(qkv, gq, gk), o1.detach())
+    # and against the oracle: restated RMSNorm.forward + naive attention, fp32
+    q, k, v = (t.float().cpu() for t in qkv.unbind(2))
+    from oracle import block_oracle as bo
+    ref = ao.base_attn(bo.rms_norm(q, gq.detach().cpu()), bo.rms_norm(k, gk.detach().cpu()), v)
+    assert ao.rel_l2(o1.detach().float().cpu(), ref) <= TOL[dtype]

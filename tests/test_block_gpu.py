@@ -135,6 +135,11 @@ def test_rmsnorm_fwd_jvp_bwd(B, L, H, D, dt, packed):
     gx, ggain = _lib.rmsnorm_bwd(gy.to(DEV), dev(x), gain.to(DEV))
     _close(gx, torch.from_numpy(cf["gx"]), _tol(dt), "gx")
     _close(ggain, torch.from_numpy(cf["ggain"]), 1e-5, "ggain")
+    # gradient written in place into one slot of a packed (B, L, 3, H, D) buffer
+    packed_grad = torch.zeros(B, L, 3, H, D, dtype=dt, device=DEV)
+    gx2, ggain2 = _lib.rmsnorm_bwd(gy.to(DEV), dev(x), gain.to(DEV), out=packed_grad[:, :, 1])
+    assert torch.equal(packed_grad[:, :, 1], gx) and torch.equal(ggain2, ggain)
+    assert float(packed_grad[:, :, 0].abs().max()) == 0 and float(packed_grad[:, :, 2].abs().max()) == 0
 
 
 def test_wrappers_under_func_jvp_and_autograd():
