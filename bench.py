@@ -37,8 +37,8 @@ MEASURED_TRAFFIC_BYTES = {"xl2_512px": 1.2129e9, "xl2_256px": 1.2125e9}
 
 WORKLOADS = {
     # name: (B, H, N, D, qk_norm)
-    "xl2_512px": (64, 16, 1024, 72, True),    # BASELINE config 4 (headline)
-    "xl2_256px": (256, 16, 256, 72, False),   # BASELINE config 3
+    "xl2_512px": (64, 16, 1024, 72, True),    # SiT/DMFT-XL/2 at 512px with qk-norm (headline)
+    "xl2_256px": (256, 16, 256, 72, False),   # SiT/DMFT-XL/2 at 256px
 }
 
 
@@ -118,7 +118,7 @@ def cpu_baseline(name, budget_s=15.0):
 
 
 def cpu_baseline_config1():
-    """BASELINE config 1 (B2 H12 N256 D64 fp32) at all cores and at the 4
+    """The CPU-runnable case (B2 H12 N256 D64 fp32) at all cores and at the 4
     intra-op threads the reference pins (train_dmf.py:33-34)."""
     import torch
     from oracle import attn_oracle as ao

@@ -69,7 +69,7 @@ def _parity(B, L, H, D, dtype, seed, std=1.0, Lkv=None, bwd=True):
         _check("dv", dv, dv_ref, tol)
 
 
-# ---- BASELINE configurations at sizes the oracle finishes in seconds -------
+# ---- benchmark configurations at sizes the oracle finishes in seconds -------
 def test_config1_fp32():
     """Config 1: B=2, H=12, N=256, D=64, fp32, N(0,1), seed 1."""
     _parity(2, 256, 12, 64, torch.float32, seed=1)
@@ -140,7 +140,7 @@ def test_packed_qkv_strided_views_match_contiguous():
             assert torch.equal(x, y)
 
 
-# ---- full BASELINE sizes through size-independent properties ---------------
+# ---- full benchmark sizes through size-independent properties ---------------
 @pytest.mark.parametrize("B,L", [(256, 256), (64, 1024)])
 def test_full_size_properties(B, L):
     """Configs 3 (B256 N256) and 4 (B64 N1024, qk-norm) at full size, bf16:

@@ -186,7 +186,7 @@ def test_fused_train_step_direct_dual_level_equals_func_jvp():
 
 @pytest.mark.gpu
 def test_dmft_b2_full_architecture_fused_graph_vs_base():
-    """BASELINE config 2 at its real architecture (DMFT-B/2: 12 blocks, hidden 768, 12 heads of 64, 256 tokens,
+    """The DMFT-B/2 forward+JVP benchmark model at its real architecture (DMFT-B/2: 12 blocks, hidden 768, 12 heads of 64, 256 tokens,
     dmf_depth 8), reduced batch: forward+JVP under bf16 autocast through the fused path replayed as a HIP graph,
     against the same weights with the naive attention and the reference's expressions run eagerly."""
     dev = "cuda:0"

@@ -143,7 +143,7 @@ def test_split_head_dim_table():
 
 
 def test_config1_fp32_oracle_is_self_consistent():
-    """BASELINE config 1 (B2 H12 N256 D64 fp32): the fp32 jvp oracle is itself
+    """The CPU-runnable benchmark case (B2 H12 N256 D64 fp32): the fp32 jvp oracle is itself
     within 1e-6 of the fp64 closed form, so a 1e-5 kernel tolerance is meaningful."""
     q, k, v, tq, tk, tv, dout = ao.make_inputs(2, 256, 12, 64, seed=1)
     o, to = ao.base_attn_jvp(q, k, v, tq, tk, tv)
