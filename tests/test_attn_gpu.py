@@ -301,3 +301,19 @@ def test_qknorm_qkvpacked_func_matches_composition(dtype):
     from oracle import block_oracle as bo
     ref = ao.base_attn(bo.rms_norm(q, gq.detach().cpu()), bo.rms_norm(k, gk.detach().cpu()), v)
     assert ao.rel_l2(o1.detach().float().cpu(), ref) <= TOL[dtype]
+
+
+def test_golden_vectors():
+    """fp32 kernels through the C ABI against the committed known-answer vectors
+    (tests/golden/attn_vectors.npz: fp64 closed forms on seeded inputs, one case with Lq != Lkv)."""
+    import os
+    import numpy as np
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "attn_vectors.npz"))
+    for n in sorted({k.split(".")[0] for k in z.files}):
+        q, k, v, tq, tk, tv, do = (torch.from_numpy(z[f"{n}.{key}"]).to(DEV) for key in ("q", "k", "v", "tq", "tk", "tv", "dout"))
+        scale = q.shape[-1] ** -0.5
+        o, to, lse, dlse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale, need_dlse=True)
+        dq, dk, dv = _lib.bwd(do, q, k, v, o, lse, scale)
+        for key, got in (("o", o), ("to", to), ("lse", lse), ("mu", dlse), ("dq", dq), ("dk", dk), ("dv", dv)):
+            err = ao.rel_l2(got.double().cpu(), torch.from_numpy(z[f"{n}.{key}"]))
+            assert err <= 1e-5, (n, key, err)

@@ -152,3 +152,20 @@ def test_config1_fp32_oracle_is_self_consistent():
     assert ao.rel_l2(to, torch.from_numpy(cf["to"])) < 2e-6
     for name, g in zip(("dq", "dk", "dv"), ao.base_attn_grads(q, k, v, dout)):
         assert ao.rel_l2(g, torch.from_numpy(cf[name])) < 2e-6
+
+
+def test_golden_vectors():
+    """The committed known-answer vectors (tests/golden/attn_vectors.npz, written once by
+    tests/golden/make_attn_vectors.py from the fp64 closed forms): the fp32 oracle -- naive
+    attention under torch.func.jvp and autograd -- must reproduce them."""
+    import os
+    import numpy as np
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "attn_vectors.npz"))
+    names = sorted({k.split(".")[0] for k in z.files})
+    assert names == ["d64", "d72_cross"]
+    for n in names:
+        q, k, v, tq, tk, tv, do = (torch.from_numpy(z[f"{n}.{key}"]) for key in ("q", "k", "v", "tq", "tk", "tv", "dout"))
+        o, to = ao.base_attn_jvp(q, k, v, tq, tk, tv)
+        dq, dk, dv = ao.base_attn_grads(q, k, v, do)
+        for key, got in (("o", o), ("to", to), ("dq", dq), ("dk", dk), ("dv", dv), ("lse", ao.lse_ref(q, k))):
+            assert ao.rel_l2(got.double(), torch.from_numpy(z[f"{n}.{key}"])) < 2e-6, (n, key)
