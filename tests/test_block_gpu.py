@@ -306,3 +306,34 @@ def test_residual_ln_modulate_wrapper_under_func_jvp_and_autograd():
     (out * dev["gy"]).sum().backward()
     for k, p, r in zip(keys, prim, bo.grads(plain, [d[k] for k in keys], d["gy"])):
         _close(p.grad, r, 2e-5, f"grad {k}")
+
+
+def test_golden_vectors():
+    """fp32 kernels through the C ABI against the committed known-answer vectors
+    (tests/golden/block_vectors.npz: fp64 closed forms on seeded inputs)."""
+    import os
+    import numpy as np
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "block_vectors.npz"))
+    g = lambda k: torch.from_numpy(z[k]).to(DEV)
+    ref = lambda k: torch.from_numpy(z[k])
+    y, ty = _lib.ln_modulate_fwd(g("x"), g("shift"), g("scale"), g("tx"), g("tshift"), g("tscale"), 1e-6, F32, True)
+    gx, gsh, gsc = _lib.ln_modulate_bwd(g("gy"), g("x"), g("scale"), 1e-6)
+    B, L, C = z["x"].shape
+    for got, key in ((y, "ln_modulate.y"), (ty, "ln_modulate.ty"), (gx, "ln_modulate.gx"),
+                     (gsh.view(B, 1, C), "ln_modulate.gshift"), (gsc.view(B, 1, C), "ln_modulate.gscale")):
+        _close(got, ref(key), 1e-5, key)
+    y, ty = _lib.gate_residual_fwd(g("x"), g("gate"), g("h"), g("tx"), g("tgate"), g("th"), True)
+    gh, gg = _lib.gate_residual_bwd(g("gy"), g("gate"), g("h"))
+    for got, key in ((y, "gate_residual.y"), (ty, "gate_residual.ty"), (gh, "gate_residual.gh"), (gg.view(B, 1, C), "gate_residual.ggate")):
+        _close(got, ref(key), 1e-5, key)
+    u = g("gelu.x")
+    y, dy = _lib.gelu_tanh_fwd(u, torch.ones_like(u))
+    _close(y, ref("gelu.y"), 1e-5, "gelu.y")
+    _close(dy, ref("gelu.dy"), 1e-5, "gelu.dy")
+    y, dy = _lib.silu_fwd(u, torch.ones_like(u))
+    _close(y, ref("silu.y"), 1e-5, "silu.y")
+    _close(dy, ref("silu.dy"), 1e-5, "silu.dy")
+    y, ty = _lib.rmsnorm_fwd(g("rms.x"), g("rms.gain"), g("rms.tx"), 1e-6, True)
+    gx, gg = _lib.rmsnorm_bwd(g("rms.gy"), g("rms.x"), g("rms.gain"))
+    for got, key in ((y, "rms.y"), (ty, "rms.ty"), (gx, "rms.gx"), (gg, "rms.ggain")):
+        _close(got, ref(key), 1e-5, key)

@@ -131,3 +131,30 @@ def test_silu_matches_library_and_derivative():
     assert torch.allclose(ty, _fd(bo.silu, (x,), (t,)), atol=1e-7)
     s = 1 / (1 + np.exp(-x.numpy()))
     assert np.allclose(ty.numpy(), s * (1 + x.numpy() * (1 - s)) * t.numpy(), atol=1e-12)
+
+
+def _golden():
+    import os
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "block_vectors.npz"))
+
+
+def test_golden_vectors():
+    """The committed known-answer vectors (tests/golden/block_vectors.npz, written once by
+    tests/golden/make_block_vectors.py from the fp64 closed forms): the torch restatements,
+    evaluated in fp64 on the stored fp32 inputs, must reproduce them."""
+    z = _golden()
+    t = lambda k: torch.from_numpy(z[k]).double()
+    close = lambda got, key, tol=1e-12: np.allclose(got.numpy(), z[key], atol=tol, rtol=tol)
+    y, ty = bo.jvp(bo.ln_modulate, (t("x"), t("shift"), t("scale")), (t("tx"), t("tshift"), t("tscale")))
+    gx, gsh, gsc = bo.grads(bo.ln_modulate, (t("x"), t("shift"), t("scale")), t("gy"))
+    assert close(y, "ln_modulate.y") and close(ty, "ln_modulate.ty", 1e-11) and close(gx, "ln_modulate.gx", 1e-11)
+    assert close(gsh, "ln_modulate.gshift", 1e-11) and close(gsc, "ln_modulate.gscale", 1e-11)
+    y, ty = bo.jvp(bo.gate_residual, (t("x"), t("gate"), t("h")), (t("tx"), t("tgate"), t("th")))
+    assert close(y, "gate_residual.y") and close(ty, "gate_residual.ty")
+    u = t("gelu.x")
+    assert close(bo.gelu_tanh(u), "gelu.y") and close(bo.silu(u), "silu.y")
+    assert close(bo.jvp(bo.gelu_tanh, (u,), (torch.ones_like(u),))[1], "gelu.dy")
+    assert close(bo.jvp(bo.silu, (u,), (torch.ones_like(u),))[1], "silu.dy")
+    y, ty = bo.jvp(lambda a: bo.rms_norm(a, t("rms.gain")), (t("rms.x"),), (t("rms.tx"),))
+    gx, gg = bo.grads(bo.rms_norm, (t("rms.x"), t("rms.gain")), t("rms.gy"))
+    assert close(y, "rms.y") and close(ty, "rms.ty", 1e-11) and close(gx, "rms.gx", 1e-11) and close(gg, "rms.ggain", 1e-11)
