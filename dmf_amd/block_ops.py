@@ -179,7 +179,7 @@ class RMSNormFunc(torch.autograd.Function):
 
 
 class DualLinearFunc(torch.autograd.Function):
-    """(x, tx, weight, bias) -> (y, ty, w) with y = x W^T + b, ty = tx W^T: exactly
+    """(x, tx, weight, bias, w_lp, b_lp) -> (y, ty, w) with y = x W^T + b, ty = tx W^T: exactly
     one library GEMM per stream.  torch's own forward-mode rule for ``linear``
     also multiplies the primal input by a materialised all-zero weight tangent
     and adds the two products (three GEMMs, two fills, a copy and an add per
@@ -188,33 +188,39 @@ class DualLinearFunc(torch.autograd.Function):
     the cast weight, is returned so that ``backward`` can reuse it)."""
 
     @staticmethod
-    def forward(x, tx, weight, bias):
+    def forward(x, tx, weight, bias, w_lp, b_lp):
         linear = torch.nn.functional.linear
         if x.is_cuda and torch.is_autocast_enabled("cuda"):
             dt = torch.get_autocast_dtype("cuda")
-            w = weight.to(dt)
-            b = None if bias is None else bias.to(dt)
+            cached = w_lp is not None and w_lp.dtype == dt
+            w = w_lp if cached else weight.to(dt)
+            b = None if bias is None else (b_lp if cached and b_lp is not None else bias.to(dt))
             with torch.autocast("cuda", enabled=False):
                 y = linear(x.to(dt), w, b)
                 ty = None if tx is None else linear(tx.to(dt), w)
-            return y, ty, (w if w is not weight else None)
+            # (an input is never handed back as an output: a cached copy reaches backward through the inputs)
+            return y, ty, (w if not cached and w is not weight else None)
         return linear(x, weight, bias), (None if tx is None else linear(tx, weight)), None
 
     @staticmethod
     def setup_context(ctx, inputs, outputs):
-        x, _, weight, bias = inputs
+        x, _, weight, bias, w_lp, _ = inputs
         w = outputs[2]
-        ctx.save_for_backward(x, weight if w is None else w)
-        ctx.weight_dtype = weight.dtype
-        ctx.bias_dtype = None if bias is None else bias.dtype
         if w is not None:
             ctx.mark_non_differentiable(w)
+        elif w_lp is not None and x.is_cuda and torch.is_autocast_enabled("cuda") and w_lp.dtype == torch.get_autocast_dtype("cuda"):
+            w = w_lp
+        else:
+            w = weight
+        ctx.save_for_backward(x, w)
+        ctx.weight_dtype = weight.dtype
+        ctx.bias_dtype = None if bias is None else bias.dtype
         ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, gy, gty, gw_unused):
         if gy is None:
-            return None, None, None, None
+            return (None,) * 6
         x, w = ctx.saved_tensors
         g2 = gy.reshape(-1, gy.shape[-1]).to(w.dtype)
         want_gx, want_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[2]
@@ -250,7 +256,7 @@ class DualLinearFunc(torch.autograd.Function):
             for t in (gw, gb):   # allocated on the side stream, consumed (and later freed) on the main one
                 if t is not None:
                     t.record_stream(main)
-        return gx, None, gw, gb
+        return gx, None, gw, gb, None, None
 
 
 _SIDE_STREAMS = {}
@@ -263,11 +269,13 @@ def _side_stream(device):
     return _SIDE_STREAMS[key]
 
 
-def dual_linear(x, weight, bias=None):
+def dual_linear(x, weight, bias=None, w_lp=None, b_lp=None):
     """``F.linear(x, weight, bias)``; a forward-AD dual ``x`` gives a dual result
-    (weight and bias are constants of the tangent map)."""
+    (weight and bias are constants of the tangent map).  ``w_lp`` / ``b_lp``: optional
+    copies of the parameters in the autocast dtype, used instead of casting per call
+    (the caller guarantees they are current)."""
     (xp,), (tx,), dual = _unpack(x)
-    y, ty, _ = _lib.run_function(DualLinearFunc, xp, tx, weight, bias)
+    y, ty, _ = _lib.run_function(DualLinearFunc, xp, tx, weight, bias, w_lp, b_lp)
     return fwAD.make_dual(y, ty) if dual else y
 
 

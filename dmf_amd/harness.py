@@ -8,6 +8,7 @@ train_dmf.py:325-330 does under bf16 autocast.
 """
 from __future__ import annotations
 
+import contextlib
 import time
 from functools import partial
 
@@ -15,6 +16,7 @@ import torch
 import torch.autograd.forward_ad as fwAD
 
 from .dmft import DMFT_models
+from .layers import frozen_low_precision_params
 
 
 def synthetic_batch(batch: int, device, seed: int = 2, input_size: int = 32, channels: int = 4, num_classes: int = 1000):
@@ -163,8 +165,11 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
                 def step(z, t, r, y, v):
                     with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
                         return model(z, t, r, y)
-            run = GraphedStep(step, *data) if graphed else step
-            sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
+            # the forward+JVP-only and no-grad passes run over frozen weights: cast them once, not per call
+            frozen = frozen_low_precision_params(model) if (mode != "train" and block_ops == "hip") else contextlib.nullcontext()
+            with frozen:
+                run = GraphedStep(step, *data) if graphed else step
+                sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
             row[f"{label}_ms_per_step"] = sec * 1e3
             row[f"{label}_images_per_s"] = batch / sec
             del model, run, step

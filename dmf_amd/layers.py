@@ -7,6 +7,7 @@ pieces (:28-29, :59-82, :158-220) that the DMFT harness needs.
 """
 from __future__ import annotations
 
+import contextlib
 import math
 from functools import partial
 
@@ -72,16 +73,36 @@ class SiLU(nn.SiLU):
 class Linear(nn.Linear):
     """``nn.Linear`` whose forward-mode pass costs one extra GEMM instead of two
     (``block_ops.dual_linear``) when ``block_ops="hip"``; parameters, state-dict
-    keys and results are those of ``nn.Linear``."""
+    keys and results are those of ``nn.Linear``.  ``lp_weight`` / ``lp_bias`` are
+    set by ``frozen_low_precision_params`` while the parameters are known not to
+    change."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, block_ops: str = "torch"):
         super().__init__(in_features, out_features, bias=bias)
         self.fused = _check_block_ops(block_ops)
+        self.lp_weight = self.lp_bias = None
 
     def forward(self, x: Tensor) -> Tensor:
         if self.fused:
-            return fused.dual_linear(x, self.weight, self.bias)
+            return fused.dual_linear(x, self.weight, self.bias, self.lp_weight, self.lp_bias)
         return super().forward(x)
+
+
+@contextlib.contextmanager
+def frozen_low_precision_params(model: nn.Module, dtype: torch.dtype = torch.bfloat16):
+    """While active, every fused ``Linear`` of ``model`` uses a copy of its parameters in
+    ``dtype`` made once on entry, instead of the per-call casts of autocast -- for loops
+    over frozen weights (sampling, evaluation, forward+JVP-only passes).  The caller must
+    not modify the parameters inside the context; results are those of autocast."""
+    layers = [m for m in model.modules() if isinstance(m, Linear) and m.fused]
+    try:
+        for m in layers:
+            m.lp_weight = m.weight.detach().to(dtype)
+            m.lp_bias = None if m.bias is None else m.bias.detach().to(dtype)
+        yield model
+    finally:
+        for m in layers:
+            m.lp_weight = m.lp_bias = None
 
 
 def modulate(x: Tensor, shift: Tensor, scale: Tensor) -> Tensor:

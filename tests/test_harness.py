@@ -229,3 +229,25 @@ def test_registry_models_fused_vs_base(name, qk_norm):
     worst = max(ao.rel_l2(p.grad.cpu(), q.grad.cpu()) for (n, p), (_, q) in zip(m.named_parameters(), m_ref.named_parameters())
                 if q.grad is not None and float(q.grad.abs().max()) > 0)
     assert worst <= 1e-3, worst
+
+
+@pytest.mark.gpu
+def test_frozen_low_precision_params_give_the_same_bits():
+    """Cached bf16 parameter copies are exactly what autocast would cast per call."""
+    from dmf_amd.layers import frozen_low_precision_params
+    dev = "cuda:0"
+    m = _small("hip", block_ops="hip", input_size=32, hidden_size=288, depth=2, num_heads=4, dmf_depth=1).to(dev)
+    m.requires_grad_(False)
+    data = harness.synthetic_batch(4, dev)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        u0, du0 = harness.meanflow_jvp(m, *data)
+        with frozen_low_precision_params(m):
+            assert m.blocks[0].attn.qkv.lp_weight.dtype == torch.bfloat16
+            u1, du1 = harness.meanflow_jvp(m, *data)
+        assert m.blocks[0].attn.qkv.lp_weight is None
+    assert torch.equal(u0, u1) and torch.equal(du0, du1)
+    # and training through cached copies still sends gradients to the fp32 parameters
+    m.requires_grad_(True)
+    with frozen_low_precision_params(m):
+        harness.train_step(m, data)
+    assert m.blocks[0].attn.qkv.weight.grad is not None and m.blocks[0].attn.qkv.weight.grad.dtype == torch.float32
