@@ -317,3 +317,24 @@ def test_golden_vectors():
         for key, got in (("o", o), ("to", to), ("lse", lse), ("mu", dlse), ("dq", dq), ("dk", dk), ("dv", dv)):
             err = ao.rel_l2(got.double().cpu(), torch.from_numpy(z[f"{n}.{key}"]))
             assert err <= 1e-5, (n, key, err)
+
+
+def test_huge_row_stride_takes_the_64bit_addressing_path():
+    """Rows 2 GiB apart: beyond the 32-bit buffer addressing of the tuned bf16 kernels, so the
+    dispatcher must hand the call to the generic kernels (64-bit pointers) -- same numbers."""
+    B, L, H, D = 1, 3, 1, 64
+    stride_l = 1 << 30                                  # elements between consecutive rows
+    cpu = [t.to(torch.bfloat16) for t in ao.make_inputs(B, L, H, D, seed=31)]
+    big = []
+    for t in cpu[:6]:
+        buf = torch.zeros((L - 1) * stride_l + D, dtype=torch.bfloat16, device=DEV)
+        view = buf.as_strided((B, L, H, D), (0, stride_l, D, 1))
+        view.copy_(t.to(DEV))
+        big.append(view)
+    q, k, v, tq, tk, tv = big
+    o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, D ** -0.5)
+    o_ref, to_ref = ao.base_attn_jvp(*[t.float() for t in cpu[:6]])
+    assert ao.rel_l2(o.float().cpu(), o_ref) <= 2e-2 and ao.rel_l2(to.float().cpu(), to_ref) <= 2e-2
+    dq, dk, dv = _lib.bwd(cpu[6].to(DEV), q, k, v, o, lse, D ** -0.5)
+    for got, ref in zip((dq, dk, dv), ao.base_attn_grads(*[t.float() for t in cpu[:3]], cpu[6].float())):
+        assert ao.rel_l2(got.float().cpu(), ref) <= 2e-2
