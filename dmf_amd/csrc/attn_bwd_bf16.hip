@@ -375,6 +375,7 @@ int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream) 
   switch (D) {
     case 64: return launch_bwd_fast_t<64>(p, BH, stream);
     case 72: return launch_bwd_fast_t<72>(p, BH, stream);
+    case 80: return launch_bwd_fast_t<80>(p, BH, stream);
     case 96: return launch_bwd_fast_t<96>(p, BH, stream);
     case 128: return launch_bwd_fast_t<128>(p, BH, stream);
     default: return 1;

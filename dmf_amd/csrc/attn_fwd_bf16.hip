@@ -390,6 +390,7 @@ int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_
   switch (D) {
     DMF_CASE(64)
     DMF_CASE(72)
+    DMF_CASE(80)
     DMF_CASE(96)
     DMF_CASE(128)
     default: return 1;
