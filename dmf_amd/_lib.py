@@ -100,6 +100,20 @@ def run_function(fn_cls, *args):
     return fn_cls.apply(*args)
 
 
+_SIDE_STREAMS = {}
+
+
+def side_stream(device) -> torch.cuda.Stream:
+    """One extra stream per device (default priority) for fork / join of independent
+    kernels; a stream capture records such a fork as parallel graph branches."""
+    key = torch.device(device).index
+    if key is None:
+        key = torch.cuda.current_device()
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return _SIDE_STREAMS[key]
+
+
 def _empty(shape, dtype, device) -> torch.Tensor:
     return _raw(torch.empty(shape, dtype=dtype, device=device))
 

@@ -232,7 +232,7 @@ class DualLinearFunc(torch.autograd.Function):
         # trick for the primal / tangent GEMMs of the forward pass measured neutral to negative and is not used).
         fork = g2.is_cuda and want_gx and (want_gw or want_gb)
         if fork:
-            main, side = torch.cuda.current_stream(g2.device), _side_stream(g2.device)
+            main, side = torch.cuda.current_stream(g2.device), _lib.side_stream(g2.device)
             side.wait_stream(main)
             torch.cuda.set_stream(side)
         try:
@@ -257,16 +257,6 @@ class DualLinearFunc(torch.autograd.Function):
                 if t is not None:
                     t.record_stream(main)
         return gx, None, gw, gb, None, None
-
-
-_SIDE_STREAMS = {}
-
-
-def _side_stream(device):
-    key = torch.device(device).index
-    if key not in _SIDE_STREAMS:
-        _SIDE_STREAMS[key] = torch.cuda.Stream(device=device)   # default priority
-    return _SIDE_STREAMS[key]
 
 
 def dual_linear(x, weight, bias=None, w_lp=None, b_lp=None):
