@@ -28,6 +28,7 @@ SIGNATURES = {
     "dmf_attn_strerror": (c_char_p, [c_int]),
     "dmf_attn_fwd_jvp": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 5 + [_F, _I, _P]),
+    "dmf_attn_fwd_qnorm": (c_int, [_P] * 7 + [_F] + [_P] * 4 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_bwd": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_block_workspace_floats": (c_int64, [_I] * 4),
     "dmf_ln_modulate_fwd": (c_int, [_P] * 8 + [_S] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
@@ -183,6 +184,45 @@ def fwd(q, k, v, scale: float, need_lse: bool = True):
             _strides(q, k, v, o), B, H, Lq, Lkv, D, float(scale), _dtype_code(q), _stream(q))
     _check(rc, "dmf_attn_fwd")
     return o, lse
+
+
+ENOKERNEL = -8   # DMF_ATTN_ENOKERNEL
+
+
+def fwd_qnorm(q, k, v, tq, tk, tv, q_gain, eps: float, scale: float, need_lse: bool = True):
+    """Forward (+ JVP when ``tq`` is given) with the per-head RMS norm of q (gain
+    ``q_gain``, fp32 (D)) applied inside the attention kernel.  Returns (o, to, lse)
+    (``to`` None without tangents), or None when no kernel implements the variant for
+    this shape / dtype -- the caller then normalises q itself."""
+    jvp = tq is not None
+    if jvp:
+        _check_inputs(q, k, v, tq, tk, tv)
+        q, k, v, tq, tk, tv = map(_prep, (q, k, v, tq, tk, tv))
+    else:
+        _check_inputs(q, k, v)
+        q, k, v = map(_prep, (q, k, v))
+    gain = _raw(q_gain)
+    if gain.dim() != 1 or gain.shape[0] != q.shape[-1] or gain.device != q.device:
+        raise ValueError("fwd_qnorm: q_gain must be a (D) tensor on the device of q")
+    gain = _raw(gain.contiguous())
+    if q.dtype != torch.bfloat16 or gain.dtype != torch.float32 or gain.data_ptr() % 16:
+        return None
+    B, Lq, H, D = q.shape
+    Lkv = k.shape[1]
+    o = _empty((B, Lq, H, D), q.dtype, q.device)
+    to = _empty((B, Lq, H, D), q.dtype, q.device) if jvp else None
+    lse = _empty((B, H, Lq), torch.float32, q.device) if (need_lse or jvp) else None
+    z = q   # stands in for absent tangents in the stride table (ignored by the library)
+    with torch.cuda.device(q.device):
+        rc = load().dmf_attn_fwd_qnorm(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _ptr(tq), _ptr(tk), _ptr(tv), gain.data_ptr(), float(eps),
+            o.data_ptr(), _ptr(to), _ptr(lse), None,
+            _strides(q, k, v, tq if jvp else z, tk if jvp else z, tv if jvp else z, o, to if jvp else o),
+            B, H, Lq, Lkv, D, float(scale), _dtype_code(q), _stream(q))
+    if rc == ENOKERNEL:
+        return None
+    _check(rc, "dmf_attn_fwd_qnorm")
+    return o, to, lse
 
 
 def bwd(dout, q, k, v, o, lse, scale: float, out=None):

@@ -229,6 +229,7 @@ int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream
     const int rc = launch_fwd_bf16_fast(p, BH, D, jvp, stream);
     if (rc != 1) return rc;   // 1 = no tuned kernel for this shape
   }
+  if (p.q_gain != nullptr) return kNoQNormKernel;   // the generic kernels take already-normalised q
   return launch_fwd_generic(p, BH, D, bf16, jvp, stream);
 }
 

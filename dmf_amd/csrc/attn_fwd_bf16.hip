@@ -46,7 +46,8 @@ struct FastCfg {
 
 // NW = waves per work-group: 4 (128 query rows, two work-groups per CU) or
 // 8 (256 query rows, one work-group per CU: half the tile traffic per FLOP).
-template <int D, bool JVP, int NW>
+// QN: per-head RMS norm of q (and its tangent) applied while the Q operands are formed.
+template <int D, bool JVP, int NW, bool QN = false>
 __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const FwdParams p) {
   constexpr int NTHR = 64 * NW, BQ = 32 * NW;
   using F = FastCfg<D>;
@@ -123,11 +124,53 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
       const uint32_t rb_tq = (uint32_t)p.st[3][1] * 2;
       load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.tq) + base(3), rb_tq, p.Lq, D * 2), rb_tq, qrow, g, dQr);
     }
+    auto lo = [](uint32_t w) { return __uint_as_float(w << 16); };
+    auto hi = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
+    if constexpr (QN) {
+      // q_hat = q r g,  dq_hat = (dq r + q dr) g  with  r = (mean q^2 + eps)^-1/2,  dr = -r^3 mean(q dq)  (models/layers.py:39-42
+      // and its tangent); this lane holds elements 16c + 8g + 0..7 of its row, the other half of the wave the rest.
+      // Rounded to bf16 before the softmax scale is applied, exactly like a separate norm kernel followed by this one.
+      float ss = 0.f, sd = 0.f;
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ss = fmaf(lo(Qr[c][e]), lo(Qr[c][e]), fmaf(hi(Qr[c][e]), hi(Qr[c][e]), ss));
+          if constexpr (JVP) sd = fmaf(lo(Qr[c][e]), lo(dQr[c][e]), fmaf(hi(Qr[c][e]), hi(dQr[c][e]), sd));
+        }
+      const float r = 1.f / sqrtf(xhalf_sum(ss) * (1.f / D) + p.q_eps);
+      const float dr = JVP ? -r * r * r * xhalf_sum(sd) * (1.f / D) : 0.f;
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) {
+        float gn[8];
+        if (2 * c + g < VPR) {
+          const f32x4* gp = reinterpret_cast<const f32x4*>(p.q_gain + 16 * c + 8 * g);
+          const f32x4 g0 = gp[0], g1 = gp[1];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            gn[e] = g0[e];
+            gn[4 + e] = g1[e];
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) gn[e] = 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float ql = lo(Qr[c][e]), qh = hi(Qr[c][e]);
+          const uint32_t qn = pack_bf16x2(ql * r * gn[2 * e], qh * r * gn[2 * e + 1]);
+          if constexpr (JVP) {
+            const uint32_t dn = pack_bf16x2(fmaf(lo(dQr[c][e]), r, ql * dr) * gn[2 * e], fmaf(hi(dQr[c][e]), r, qh * dr) * gn[2 * e + 1]);
+            dQr[c][e] = dn;
+          }
+          Qr[c][e] = qn;
+        }
+      }
+    }
     auto scaled = [&](u32x4 x) {
       u32x4 y;
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        y[e] = pack_bf16x2(__uint_as_float(x[e] << 16) * p.scale, __uint_as_float(x[e] & 0xffff0000u) * p.scale);
+      for (int e = 0; e < 4; ++e) y[e] = pack_bf16x2(lo(x[e]) * p.scale, hi(x[e]) * p.scale);
       return y;
     };
 #pragma unroll
@@ -353,18 +396,27 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
                                          [&](int t, int i) { return fmaf(-mu_n, O[t][i] * inv_l, dO[t][i] * inv_l); }, tail_to);
 }
 
-template <int D, bool JVP, int NW>
-static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
+template <int D, bool JVP, int NW, bool QN>
+static int launch_fast_q(const FwdParams& p, int BH, hipStream_t stream) {
   using F = FastCfg<D>;
   constexpr int tiles = 2 * (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES) + 512;
   constexpr int stage = 32 * NW * Cfg<__bf16, D>::OROWV * 16;
   constexpr int smem = tiles > stage ? tiles : stage;
-  auto kern = attn_fwd_bf16_kernel<D, JVP, NW>;
+  auto kern = attn_fwd_bf16_kernel<D, JVP, NW, QN>;
   static bool lds_ok[64] = {};
   if (!ensure_dynamic_lds(kern, smem, lds_ok)) return -7;
   const uint32_t nqb = (p.Lq + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(64 * NW), smem, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+template <int D, bool JVP, int NW>
+static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
+  if (p.q_gain != nullptr) {
+    if (reinterpret_cast<uintptr_t>(p.q_gain) % 16) return -6;
+    return launch_fast_q<D, JVP, NW, true>(p, BH, stream);
+  }
+  return launch_fast_q<D, JVP, NW, false>(p, BH, stream);
 }
 
 // Work-group width policy (256-row work-groups when the sequence fills them).

@@ -16,7 +16,13 @@ struct FwdParams {
   int64_t st[8][3];         // q, k, v, tq, tk, tv, o, to
   int H, Lq, Lkv;
   float scale, scale_log2;  // softmax scale and scale * log2(e)
+  // Optional per-head RMS norm of q (and of its tangent) folded into the kernel's Q load: gain (D) fp32, or
+  // nullptr.  Only the tuned bf16 kernels implement it; the dispatcher reports kNoQNormKernel otherwise.
+  const float* q_gain;
+  float q_eps;
 };
+
+constexpr int kNoQNormKernel = -8;
 
 struct BwdParams {
   const void *dout, *q, *k, *v, *o;

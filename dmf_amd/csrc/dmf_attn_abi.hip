@@ -47,13 +47,17 @@ const char* dmf_attn_strerror(int code) {
     case DMF_ATTN_ENULL: return "a required pointer is NULL";
     case DMF_ATTN_EALIGN: return "a base pointer is not 16-byte aligned";
     case DMF_ATTN_ELAUNCH: return "the HIP runtime rejected the kernel launch";
+    case DMF_ATTN_ENOKERNEL: return "no kernel implements this variant for the given shape / dtype";
     default: return "unknown error code";
   }
 }
 
+static_assert(dmf::kNoQNormKernel == DMF_ATTN_ENOKERNEL, "dispatcher code and ABI code must agree");
+
 static int fwd_impl(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,
                     void* o, void* to, float* lse, float* dlse, const int64_t* strides, bool jvp,
-                    int B, int H, int Lq, int Lkv, int D, float scale, int dtype, void* stream) {
+                    int B, int H, int Lq, int Lkv, int D, float scale, int dtype, void* stream,
+                    const float* q_gain = nullptr, float q_eps = 0.f) {
   if (int rc = check_common(B, H, Lq, Lkv, D, dtype)) return rc;
   if (strides == nullptr) return DMF_ATTN_ENULL;
   const int eb = dtype == DMF_ATTN_BF16 ? 2 : 4;
@@ -63,16 +67,31 @@ static int fwd_impl(const void* q, const void* k, const void* v, const void* tq,
   const int slots_jvp[8] = {0, 1, 2, 3, 4, 5, 6, 7};
   const int slots_fwd[4] = {0, 1, 2, 6};
   const int n = jvp ? 8 : 4;
+  // the q-norm entry point always passes the 8-tensor stride table
+  const bool wide = jvp || q_gain != nullptr;
   for (int i = 0; i < n; ++i) {
     const int slot = jvp ? slots_jvp[i] : slots_fwd[i];
-    if (int rc = check_tensor(ptrs[slot], strides + 4 * i, eb, p.st[slot])) return rc;
+    if (int rc = check_tensor(ptrs[slot], strides + 4 * (wide ? slot : i), eb, p.st[slot])) return rc;
   }
   if (jvp && lse == nullptr) return DMF_ATTN_ENULL;
   if (lse != nullptr && reinterpret_cast<uintptr_t>(lse) % 4) return DMF_ATTN_EALIGN;
   p.q = q; p.k = k; p.v = v; p.tq = tq; p.tk = tk; p.tv = tv; p.o = o; p.to = to; p.lse = lse; p.dlse = dlse;
   p.H = H; p.Lq = Lq; p.Lkv = Lkv;
   p.scale = scale; p.scale_log2 = scale * 1.4426950408889634f;
+  p.q_gain = q_gain; p.q_eps = q_eps;
   return dmf::launch_fwd(p, B * H, D, dtype == DMF_ATTN_BF16, jvp, static_cast<hipStream_t>(stream));
+}
+
+int dmf_attn_fwd_qnorm(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,
+                       const float* q_gain, float q_eps, void* o, void* to, float* lse, float* dlse,
+                       const int64_t* strides, int B, int H, int Lq, int Lkv, int D, float scale, int dtype,
+                       void* stream) {
+  if (q_gain == nullptr) return DMF_ATTN_ENULL;
+  if (reinterpret_cast<uintptr_t>(q_gain) % 16) return DMF_ATTN_EALIGN;
+  const bool jvp = to != nullptr;
+  if (!jvp) tq = tk = tv = nullptr, dlse = nullptr;
+  return fwd_impl(q, k, v, tq, tk, tv, o, to, lse, dlse, strides, jvp, B, H, Lq, Lkv, D, scale, dtype, stream, q_gain,
+                  q_eps);
 }
 
 int dmf_attn_fwd_jvp(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,

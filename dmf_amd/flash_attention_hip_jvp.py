@@ -167,14 +167,21 @@ def flash_attn_qkvpacked_func(qkv, softmax_scale=None):
     return out if tg is None else fwAD.make_dual(out, t_out)
 
 
+# Normalise q inside the attention kernel where a kernel offers it (module switch for A/B timing and tests).
+IN_KERNEL_Q_NORM = True
+
+
 class QKNormAttnQKVPackedFunc(torch.autograd.Function):
     """(qkv, tqkv, q_gain, k_gain, eps, softmax_scale) -> (o, lse, to): per-head RMS
     norm of the q and k slots of a packed (B, L, 3, H, D) projection output followed
     by attention -- ``q, k = self.q_norm(q), self.k_norm(k); x = self.attn(q, k, v)``
     (reference models/layers.py:147-151) -- as one autograd node.  Forward is the
-    fused RMS-norm kernel (primal + tangent) on each slot, read in place, then the
-    attention kernel; backward sends dv and the two norm gradients straight into the
-    three slots of one packed gradient buffer."""
+    fused RMS-norm kernel (primal + tangent) on the k slot, read in place, then the
+    attention kernel, which normalises q (and its tangent) itself while loading it;
+    where no kernel offers that (fp32, untuned shapes) the q slot goes through the
+    RMS-norm kernel as well.  Backward sends dv and the two norm gradients straight
+    into the three slots of one packed gradient buffer.  ``qn`` is None when q was
+    normalised inside the attention kernel (backward then recomputes it)."""
 
     @staticmethod
     def forward(qkv, tqkv, q_gain, k_gain, eps, softmax_scale):
@@ -182,8 +189,12 @@ class QKNormAttnQKVPackedFunc(torch.autograd.Function):
         scale = _default_scale(q, softmax_scale)
         jvp = tqkv is not None
         tq, tk, tv = tqkv.unbind(2) if jvp else (None, None, None)
-        qn, tqn = _lib.rmsnorm_fwd(q, q_gain, tq, eps, jvp)
         kn, tkn = _lib.rmsnorm_fwd(k, k_gain, tk, eps, jvp)
+        fused = _lib.fwd_qnorm(q, kn, v, tq, tkn, tv, q_gain, eps, scale) if IN_KERNEL_Q_NORM else None
+        if fused is not None:
+            o, to, lse = fused
+            return o, lse, to, None, kn
+        qn, tqn = _lib.rmsnorm_fwd(q, q_gain, tq, eps, jvp)
         if jvp:
             o, to, lse = _lib.fwd_jvp(qn, kn, v, tqn, tkn, tv, scale)
         else:
@@ -196,7 +207,7 @@ class QKNormAttnQKVPackedFunc(torch.autograd.Function):
         qkv, _, q_gain, k_gain, eps, softmax_scale = inputs
         o, lse, _, qn, kn = outputs
         ctx.save_for_backward(qkv, q_gain, k_gain, qn, kn, o, lse)
-        ctx.mark_non_differentiable(qn, kn)
+        ctx.mark_non_differentiable(*(t for t in (qn, kn) if t is not None))
         ctx.eps, ctx.softmax_scale = eps, _default_scale(qkv, softmax_scale)
         ctx.set_materialize_grads(False)
 
@@ -206,6 +217,8 @@ class QKNormAttnQKVPackedFunc(torch.autograd.Function):
             return (None,) * 6
         qkv, q_gain, k_gain, qn, kn, o, lse = ctx.saved_tensors
         q, k, v = qkv.unbind(2)
+        if qn is None:
+            qn, _ = _lib.rmsnorm_fwd(q, q_gain, None, ctx.eps, False)
         gqkv = torch.empty(qkv.shape, dtype=qkv.dtype, device=qkv.device)
         gq, gk, gv = gqkv.unbind(2)
         dqn = torch.empty(qn.shape, dtype=qn.dtype, device=qn.device)

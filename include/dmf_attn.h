@@ -57,7 +57,8 @@ enum {
   DMF_ATTN_ESTRIDE = -4,   /* last-dim stride != 1 or a stride breaks alignment */
   DMF_ATTN_ENULL = -5,     /* a required pointer is NULL                        */
   DMF_ATTN_EALIGN = -6,    /* a base pointer is not 16-byte aligned             */
-  DMF_ATTN_ELAUNCH = -7    /* the HIP runtime rejected the launch               */
+  DMF_ATTN_ELAUNCH = -7,   /* the HIP runtime rejected the launch               */
+  DMF_ATTN_ENOKERNEL = -8  /* no kernel implements this variant for the given shape / dtype; nothing was launched */
 };
 
 /* Library version, (major << 16) | minor. */
@@ -94,6 +95,32 @@ DMF_ATTN_API int dmf_attn_fwd(const void* q, const void* k, const void* v,
                  const int64_t* strides,
                  int B, int H, int Lq, int Lkv, int D,
                  float scale, int dtype, void* stream);
+
+/*
+ * Forward (+ JVP when `to` is given) with the per-head RMS norm of q folded into
+ * the kernel's Q load, so that normalised q (and its tangent) never travel
+ * through HBM:
+ *   r = rsqrt(mean_d(q^2) + q_eps),  q_hat = q r gain,
+ *   tq_hat = (tq r + q dr) gain,  dr = -r^3 mean_d(q tq),
+ * then attention on (q_hat, k, v) and tangents (tq_hat, tk, tv) as above; q_hat
+ * and tq_hat are rounded to `dtype` before use, like the outputs of
+ * dmf_rmsnorm_fwd (dmf_block.h).  Replaces `q = self.q_norm(q)` together with
+ * the attention call that follows it (models/layers.py:148-151); k is read as
+ * given (already normalised: each k row is shared by every q row, so its norm
+ * stays a separate pass).  q_gain: (D) fp32, 16-byte aligned.
+ * strides: 8 tensors {q, k, v, tq, tk, tv, o, to}; with to == NULL (primal
+ * only) tq, tk, tv, dlse and their strides are ignored and lse may be NULL.
+ * Only the tuned bf16 kernels implement this variant: DMF_ATTN_ENOKERNEL is
+ * returned (and nothing launched) for fp32 or for a shape they do not cover --
+ * the caller then normalises q itself and calls dmf_attn_fwd[_jvp].
+ */
+DMF_ATTN_API int dmf_attn_fwd_qnorm(const void* q, const void* k, const void* v,
+                     const void* tq, const void* tk, const void* tv,
+                     const float* q_gain, float q_eps,
+                     void* o, void* to, float* lse, float* dlse,
+                     const int64_t* strides,
+                     int B, int H, int Lq, int Lkv, int D,
+                     float scale, int dtype, void* stream);
 
 /*
  * Backward on the primal output: dQ, dK, dV from (dout, q, k, v, o, lse).

@@ -266,12 +266,14 @@ def test_qkvpacked_func_matches_unpacked_and_writes_packed_grads(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_qknorm_qkvpacked_func_matches_composition(dtype):
-    """RMS-norm of the q / k slots + attention as one node on the packed buffer: same
-    kernels as rms_norm -> rms_norm -> flash_attn_func on the slices, so the same bits
-    for outputs, tangents and the packed gradient (which the kernels fill in place)."""
+def test_qknorm_qkvpacked_func_matches_composition(dtype, monkeypatch):
+    """RMS-norm of the q / k slots + attention as one node on the packed buffer: with
+    the in-kernel q norm switched off, the same kernels as rms_norm -> rms_norm ->
+    flash_attn_func on the slices, so the same bits for outputs, tangents and the
+    packed gradient (which the kernels fill in place)."""
     import dmf_amd
-    from dmf_amd import block_ops
+    from dmf_amd import block_ops, flash_attention_hip_jvp
+    monkeypatch.setattr(flash_attention_hip_jvp, "IN_KERNEL_Q_NORM", False)
     B, L, H, D = 2, 136, 3, 72
     g = torch.Generator().manual_seed(23)
     qkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(DEV)
@@ -301,6 +303,98 @@ def test_qknorm_qkvpacked_func_matches_composition(dtype):
     from oracle import block_oracle as bo
     ref = ao.base_attn(bo.rms_norm(q, gq.detach().cpu()), bo.rms_norm(k, gk.detach().cpu()), v)
     assert ao.rel_l2(o1.detach().float().cpu(), ref) <= TOL[dtype]
+
+
+QNORM_SHAPES = [  # B, Lq, Lkv, H, D
+    (2, 136, 136, 3, 72), (1, 1024, 1024, 2, 72), (2, 256, 256, 4, 64), (1, 300, 300, 2, 128), (1, 200, 200, 2, 80),
+    (1, 64, 64, 2, 64), (1, 100, 100, 2, 96), (1, 77, 333, 2, 72), (1, 1, 5, 1, 64),
+]
+
+
+@pytest.mark.parametrize("shape", QNORM_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("jvp", [True, False], ids=["jvp", "primal"])
+def test_fwd_qnorm_matches_separate_norm_and_oracle(shape, jvp):
+    """q normalised inside the attention kernel against (a) the separate RMS-norm kernel
+    followed by the plain attention kernel -- same per-element formulas, only the order of
+    the sum of squares differs, so agreement at rounding level -- and (b) the fp32 oracle:
+    restated RMSNorm.forward (models/layers.py:39-42), its forward-mode tangent by
+    torch.func.jvp, and naive attention."""
+    from oracle import block_oracle as bo
+    B, Lq, Lkv, H, D = shape
+    g = torch.Generator().manual_seed(101 + D + Lq)
+    mk = lambda L: torch.randn(B, L, H, D, generator=g).to(torch.bfloat16)
+    q, tq, k, tk, v, tv = mk(Lq), mk(Lq), mk(Lkv), mk(Lkv), mk(Lkv), mk(Lkv)
+    q = q * (0.25 + 4 * torch.rand(B, Lq, H, 1, generator=g)).to(torch.bfloat16)   # rows of very different norms
+    gain = 1 + 0.3 * torch.randn(D, generator=g)
+    eps, scale = 1e-6, D ** -0.5
+    d = lambda t: t.to(DEV)
+    got = _lib.fwd_qnorm(d(q), d(k), d(v), *((d(tq), d(tk), d(tv)) if jvp else (None, None, None)), d(gain), eps, scale)
+    assert got is not None, "the tuned bf16 kernels cover every shape in this list"
+    o, to, lse = got
+    qn, tqn = _lib.rmsnorm_fwd(d(q), d(gain), d(tq) if jvp else None, eps, jvp)
+    if jvp:
+        o2, to2, lse2 = _lib.fwd_jvp(qn, d(k), d(v), tqn, d(tk), d(tv), scale)
+        assert ao.rel_l2(to.float(), to2.float()) <= 3e-3
+    else:
+        o2, lse2 = _lib.fwd(qn, d(k), d(v), scale)
+        assert to is None
+    assert ao.rel_l2(o.float(), o2.float()) <= 3e-3 and ao.rel_l2(lse, lse2) <= 1e-3
+    f = lambda t: t.float()
+    if jvp:
+        qn_ref, tqn_ref = bo.jvp(lambda x: bo.rms_norm(x, gain, eps), (f(q),), (f(tq),))
+        o_ref, to_ref = ao.base_attn_jvp(qn_ref, f(k), f(v), tqn_ref, f(tk), f(tv))
+        assert ao.rel_l2(to.float().cpu(), to_ref) <= TOL[torch.bfloat16]
+    else:
+        o_ref = ao.base_attn(bo.rms_norm(f(q), gain, eps), f(k), f(v))
+    assert ao.rel_l2(o.float().cpu(), o_ref) <= TOL[torch.bfloat16]
+
+
+def test_fwd_qnorm_reports_no_kernel_for_fp32_and_bad_gain():
+    q = torch.randn(1, 40, 2, 64, device=DEV)
+    gain = torch.ones(64, device=DEV)
+    assert _lib.fwd_qnorm(q, q, q, None, None, None, gain, 1e-6, 0.125) is None
+    h = torch.randn(1, 40, 2, 32, device=DEV).bfloat16()                          # head dim 32: generic kernels only
+    assert _lib.fwd_qnorm(h, h, h, None, None, None, gain[:32].clone(), 1e-6, 0.125) is None
+    lib = _lib.load()
+    st = _lib._strides(*([q] * 8))
+    args = lambda gp: (q.data_ptr(), q.data_ptr(), q.data_ptr(), None, None, None, gp, 1e-6, q.data_ptr(), None, None, None,
+                       st, 1, 2, 40, 40, 64, 0.125, 0, None)
+    assert lib.dmf_attn_fwd_qnorm(*args(gain.data_ptr())) == _lib.ENOKERNEL      # fp32: no kernel, nothing launched
+    assert lib.dmf_attn_fwd_qnorm(*args(None)) == -5                               # NULL gain
+    assert lib.dmf_attn_fwd_qnorm(*args(gain.data_ptr() + 4)) == -6                # misaligned gain
+    assert b"no kernel" in lib.dmf_attn_strerror(_lib.ENOKERNEL)
+
+
+def test_qknorm_qkvpacked_in_kernel_q_norm():
+    """The packed q/k-norm + attention node with q normalised inside the attention kernel
+    (bf16): outputs, tangents and gradients against the composition of separate ops at
+    rounding level, under torch.func.jvp, with backward (which recomputes q_hat), and no-grad."""
+    import dmf_amd
+    from dmf_amd import block_ops, flash_attention_hip_jvp
+    assert flash_attention_hip_jvp.IN_KERNEL_Q_NORM
+    B, L, H, D = 2, 264, 3, 72
+    g = torch.Generator().manual_seed(29)
+    qkv = torch.randn(B, L, 3, H, D, generator=g).to(torch.bfloat16).to(DEV)
+    tqkv = torch.randn(B, L, 3, H, D, generator=g).to(torch.bfloat16).to(DEV)
+    dout = torch.randn(B, L, H, D, generator=g).to(torch.bfloat16).to(DEV)
+    gq = (1 + 0.2 * torch.randn(D, generator=g)).to(DEV).requires_grad_()
+    gk = (1 + 0.2 * torch.randn(D, generator=g)).to(DEV).requires_grad_()
+    gq2, gk2 = gq.detach().clone().requires_grad_(), gk.detach().clone().requires_grad_()
+    a, b = qkv.clone().requires_grad_(), qkv.clone().requires_grad_()
+
+    def composed(x):
+        q, k, v = x.unbind(2)
+        return dmf_amd.flash_attn_func(block_ops.rms_norm(q, gq2), block_ops.rms_norm(k, gk2), v)
+
+    o1, to1 = torch.func.jvp(lambda x: dmf_amd.flash_attn_qknorm_qkvpacked_func(x, gq, gk), (a,), (tqkv,))
+    o2, to2 = torch.func.jvp(composed, (b,), (tqkv,))
+    r = lambda x, y: ao.rel_l2(x.float(), y.float())
+    assert r(o1, o2) <= 3e-3 and r(to1, to2) <= 3e-3
+    o1.backward(dout)
+    o2.backward(dout)
+    assert r(a.grad, b.grad) <= 5e-3 and r(gq.grad, gq2.grad) <= 5e-3 and r(gk.grad, gk2.grad) <= 5e-3
+    with torch.no_grad():
+        assert torch.equal(dmf_amd.flash_attn_qknorm_qkvpacked_func(qkv, gq, gk), o1.detach())
 
 
 def test_golden_vectors():
