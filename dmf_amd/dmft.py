@@ -47,6 +47,55 @@ class PatchEmbed(nn.Module):
         return block_ops_mod.dual_linear(patches, self.proj.weight.reshape(self.proj.out_channels, -1), self.proj.bias)
 
 
+def chained_blocks(blocks, conds, final_layer, c_final, x, tap=None):
+    """A stack of DiT blocks and the final layer in fused mode: same values as the
+    plain loop ``for blk, c in zip(blocks, conds): x = blk(x, c)`` followed by
+    ``final_layer(x, c_final)`` (before unpatchify), but every gated residual is
+    computed by the kernel that also normalises and modulates the result for its
+    consumer (the block's own MLP branch, the next block's attention branch, or the
+    final layer), so the residual stream is read and written once per half block.
+    ``tap(i, x)`` is called with the residual stream after block ``i``."""
+    mods = [blk.adaLN_modulation(c).chunk(6, dim=-1) for blk, c in zip(blocks, conds)]
+    f_shift, f_scale = final_layer.adaLN_modulation(c_final).chunk(2, dim=-1)
+    z = block_ops_mod.ln_modulate(x, mods[0][0], mods[0][1], blocks[0].norm1.eps)
+    for i, blk in enumerate(blocks):
+        if i + 1 < len(blocks):
+            nxt = (mods[i + 1][0], mods[i + 1][1], blocks[i + 1].norm1.eps)
+        else:
+            nxt = (f_shift, f_scale, final_layer.norm_final.eps)
+        x, z = blk.forward_chained(x, z, mods[i], *nxt)
+        if tap is not None:
+            tap(i, x)
+    return final_layer.linear(z)
+
+
+def unpatchify(x: Tensor, channels: int, patch: int) -> Tensor:
+    """(B, L, p*p*C) tokens -> (B, C, H, W) image (reference models/dmft.py:116-124, models/sit.py:122-129)."""
+    h = w = int(x.shape[1] ** 0.5)
+    assert h * w == x.shape[1]
+    x = x.reshape(x.shape[0], h, w, patch, patch, channels)
+    x = torch.einsum("nhwpqc->nchpwq", x)
+    return x.reshape(x.shape[0], channels, h * patch, w * patch)
+
+
+def trunc_normal_init_(model: nn.Module, std: float = 0.02, seed: int = 0) -> nn.Module:
+    """Benchmark initialisation: every weight matrix / embedding ~ truncated
+    N(0, std) (cut at 2 std), biases zero.  With the reference's zero-gate
+    initialisation attention contributes nothing to the output, so timing and
+    parity runs use this instead."""
+    g = torch.Generator().manual_seed(seed)
+    for name, prm in model.named_parameters():
+        if name == "pos_embed":
+            continue
+        if prm.dim() >= 2:
+            w = torch.empty(prm.shape, dtype=torch.float32)
+            nn.init.trunc_normal_(w, std=std, a=-2 * std, b=2 * std, generator=g)
+            prm.data.copy_(w)
+        elif name.endswith("bias"):
+            prm.data.zero_()
+    return model
+
+
 class DMFT(nn.Module):
     """Reference models/dmft.py:27-151."""
 
@@ -105,47 +154,14 @@ class DMFT(nn.Module):
             nn.init.constant_(self.logvar_linear.bias, 0)
 
     def init_trunc_normal_(self, std: float = 0.02, seed: int = 0) -> "DMFT":
-        """Benchmark initialisation: every weight matrix / embedding ~ truncated
-        N(0, std) (cut at 2 std), biases zero.  With the reference's zero-gate
-        initialisation attention contributes nothing to the output, so timing and
-        parity runs use this instead."""
-        g = torch.Generator().manual_seed(seed)
-        for name, prm in self.named_parameters():
-            if name == "pos_embed":
-                continue
-            if prm.dim() >= 2:
-                w = torch.empty(prm.shape, dtype=torch.float32)
-                nn.init.trunc_normal_(w, std=std, a=-2 * std, b=2 * std, generator=g)
-                prm.data.copy_(w)
-            elif name.endswith("bias"):
-                prm.data.zero_()
-        return self
+        return trunc_normal_init_(self, std, seed)
 
     def unpatchify(self, x: Tensor) -> Tensor:
-        c, p = self.out_channels, self.patch_size
-        h = w = int(x.shape[1] ** 0.5)
-        assert h * w == x.shape[1]
-        x = x.reshape(x.shape[0], h, w, p, p, c)
-        x = torch.einsum("nhwpqc->nchpwq", x)
-        return x.reshape(x.shape[0], c, h * p, w * p)
+        return unpatchify(x, self.out_channels, self.patch_size)
 
     def _forward_chained(self, x, c_t, c_r):
-        """The block stack and final layer in fused mode: same values as the plain
-        loop, but every gated residual is computed by the kernel that also
-        normalises and modulates the result for its consumer (the block's own MLP
-        branch, the next block's attention branch, or the final layer), so the
-        residual stream is read and written once per half block."""
         conds = [c_t] * self.dmf_depth + [c_r] * (len(self.blocks) - self.dmf_depth)
-        mods = [blk.adaLN_modulation(c).chunk(6, dim=-1) for blk, c in zip(self.blocks, conds)]
-        f_shift, f_scale = self.final_layer.adaLN_modulation(c_r).chunk(2, dim=-1)
-        z = block_ops_mod.ln_modulate(x, mods[0][0], mods[0][1], self.blocks[0].norm1.eps)
-        for i, blk in enumerate(self.blocks):
-            if i + 1 < len(self.blocks):
-                nxt = (mods[i + 1][0], mods[i + 1][1], self.blocks[i + 1].norm1.eps)
-            else:
-                nxt = (f_shift, f_scale, self.final_layer.norm_final.eps)
-            x, z = blk.forward_chained(x, z, mods[i], *nxt)
-        return self.final_layer.linear(z)
+        return chained_blocks(self.blocks, conds, self.final_layer, c_r, x)
 
     def forward(self, x, t, r, y, return_logvar: bool = False):
         t, r = t.reshape(-1), r.reshape(-1)

@@ -4,11 +4,17 @@
 (loss.py:165-173): ``torch.func.jvp`` through the whole model with tangents
 (v, 1, 0) for (x_t, t, r), target ``u_tgt = v + (r - t) * du/dt`` detached.
 ``train_step`` adds the backward on the primal output only, as
-train_dmf.py:325-330 does under bf16 autocast.
+train_dmf.py:325-330 does under bf16 autocast.  ``dmf_loss`` restates the whole
+training loss around that site (loss.py:142-181: the flow-matching branch with
+gradients, the guidance calls without, the JVP branch, log-variance weighting),
+``fm_loss`` the flow-matching loss that ``train_fm.py`` trains SiT with
+(loss.py:208-231); both take their random draws as arguments, so a step is a pure
+function of tensors and can be captured into a HIP graph.
 """
 from __future__ import annotations
 
 import contextlib
+import math
 import time
 from functools import partial
 
@@ -17,6 +23,7 @@ import torch.autograd.forward_ad as fwAD
 
 from .dmft import DMFT_models
 from .layers import frozen_low_precision_params
+from .sit import SiT_models
 
 
 def synthetic_batch(batch: int, device, seed: int = 2, input_size: int = 32, channels: int = 4, num_classes: int = 1000):
@@ -63,12 +70,136 @@ def train_step(model, batch, autocast: bool = True, functorch: bool = True):
     return loss
 
 
+def interpolant(x, t, eps, path_type: str = "linear"):
+    """(x_t, v_t) of the noising path (loss.py:7-23) for the noise ``eps``."""
+    if path_type == "linear":
+        alpha, sigma, d_alpha, d_sigma = 1 - t, t, -1, 1
+    elif path_type == "cosine":
+        alpha, sigma = torch.cos(t * math.pi / 2), torch.sin(t * math.pi / 2)
+        d_alpha, d_sigma = (-math.pi / 2) * torch.sin(t * math.pi / 2), (math.pi / 2) * torch.cos(t * math.pi / 2)
+    else:
+        raise NotImplementedError(path_type)
+    return alpha * x + sigma * eps, d_alpha * x + d_sigma * eps
+
+
+def _per_sample(err, reduce):
+    return reduce(err, dim=list(range(1, err.dim())))
+
+
+def log_lv_loss(x, y, lv, eps: float = 0.01):
+    """(sum of squares, log-variance weighted loss) per sample -- loss.py:30-35."""
+    err = (x - y) ** 2
+    mean = _per_sample(err, torch.mean)
+    return _per_sample(err, torch.sum), torch.log((1 / lv.exp()) * mean + eps) + lv
+
+
+def mse_loss(x, y):
+    """(sum of squares, mean of squares) per sample -- loss.py:38-42."""
+    err = (x - y) ** 2
+    return _per_sample(err, torch.sum), _per_sample(err, torch.mean)
+
+
+def compute_guidance(model, x, t, y, v_t, drop_ids, omega: float = 0.5, g_min: float = 0.0, g_max: float = 1.0,
+                     g_type: str = "default", null_class: int = 1000):
+    """Guided regression target (loss.py:57-86).  ``"mg"`` calls the trained model
+    itself as ``model(x, t, t, y)``, ``"distill"`` a frozen single-time teacher as
+    ``model(x, t, y)`` -- both without gradients on a 2B batch (conditional and
+    unconditional halves), which is the primal-only, lse-free mode of the operator."""
+    if g_type == "default":
+        return v_t
+    if g_type not in ("mg", "distill"):
+        raise NotImplementedError(f"Unknown guidance type: {g_type}")
+    in_range = (t >= g_min) & (t <= g_max)
+    with torch.no_grad():
+        x_2, t_2 = torch.cat([x, x], dim=0), torch.cat([t, t], dim=0)
+        y_2 = torch.cat([y, torch.full_like(y, null_class)], dim=0)
+        v = (model(x_2, t_2, t_2, y_2) if g_type == "mg" else model(x_2, t_2, y_2)).to(torch.float32)
+        v_cond, v_uncond = v.chunk(2, dim=0)
+    if g_type == "mg":
+        return torch.where(in_range & (~drop_ids.reshape(-1, 1, 1, 1)), v_t + omega * (v_cond - v_uncond), v_t)
+    return torch.where(in_range, v_uncond + omega * (v_cond - v_uncond), v_cond)   # no class dropout for distillation
+
+
+def dmf_loss(model, x, y, drop_ids, t_fm, t_mf, r_mf, eps_fm, eps_mf, model_t=None, functorch: bool = True,
+             path_type: str = "linear", **guidance):
+    """Per-sample training loss of ``DMFLoss.__call__`` (loss.py:142-181) and its
+    dictionary of parts.  ``y`` already carries the dropped labels and ``drop_ids``
+    says which (``cond_drop``, loss.py:129-133); times are (B, 1, 1, 1) and the two
+    noise tensors shaped like ``x`` (``sample_times`` / ``interpolant`` draw them in
+    the reference).  ``model`` must have a log-variance head.  Four model calls:
+    flow-matching branch with gradients, two guidance evaluations without (on
+    ``model_t``, default ``model``), and the MeanFlow branch under forward-mode AD
+    with tangents (v_tgt, 1, 0), whose target is detached."""
+    model_t = model if model_t is None else model_t
+    x_t_fm, v_t_fm = interpolant(x, t_fm, eps_fm, path_type)
+    v_fm, lv_fm = model(x_t_fm, t_fm, t_fm, y, return_logvar=True)
+    v_tgt_fm = compute_guidance(model_t, x_t_fm, t_fm, y, v_t_fm, drop_ids, **guidance).detach()
+    fm_mse, fm_lp = log_lv_loss(v_fm, v_tgt_fm, lv_fm)
+
+    x_t_mf, v_t_mf = interpolant(x, t_mf, eps_mf, path_type)
+    v_tgt_mf = compute_guidance(model_t, x_t_mf, t_mf, y, v_t_mf, drop_ids, **guidance).detach()
+    tangents = (v_tgt_mf, torch.ones_like(t_mf), torch.zeros_like(r_mf))
+    if functorch:
+        (u, lv_mf), (du_dt, _) = torch.func.jvp(partial(model, y=y, return_logvar=True), (x_t_mf, t_mf, r_mf), tangents)
+    else:
+        with fwAD.dual_level():
+            out, lv = model(*(fwAD.make_dual(p, tg) for p, tg in zip((x_t_mf, t_mf, r_mf), tangents)), y, return_logvar=True)
+            (u, du_dt), lv_mf = fwAD.unpack_dual(out), fwAD.unpack_dual(lv).primal
+    u_tgt = (v_tgt_mf + (r_mf - t_mf) * du_dt).detach()
+    mf_mse, mf_lp = log_lv_loss(u, u_tgt, lv_mf)
+    return 0.5 * (fm_lp + mf_lp), {"fm_loss": fm_mse, "fm_p_loss": fm_lp, "mf_p_loss": mf_lp, "mf_loss": mf_mse}
+
+
+def fm_loss(model, x, y, t, eps, path_type: str = "linear"):
+    """Per-sample flow-matching loss of ``FMLoss.__call__`` without the projection
+    term (loss.py:224-230): ``model`` is a single-time (SiT) model."""
+    x_t, v_t = interpolant(x, t, eps, path_type)
+    fm, loss = mse_loss(model(x_t, t, y), v_t)
+    return loss, {"fm_loss": fm}
+
+
+def dmf_train_step(model, batch, model_t=None, functorch: bool = True, **guidance):
+    """One optimisation step's forward and backward as train_dmf.py:325-330 runs
+    them: ``dmf_loss`` under bf16 autocast, mean over the batch, backward."""
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        loss, _ = dmf_loss(model, *batch, model_t=model_t, functorch=functorch, **guidance)
+    loss = loss.mean()
+    loss.backward()
+    return loss
+
+
+def fm_train_step(model, batch):
+    """train_fm.py:347-352: ``fm_loss`` under bf16 autocast, mean, backward."""
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        loss, _ = fm_loss(model, *batch)
+    loss = loss.mean()
+    loss.backward()
+    return loss
+
+
+def synthetic_loss_batch(batch: int, device, seed: int = 3, input_size: int = 32, channels: int = 4, num_classes: int = 1000,
+                         cfg_prob: float = 0.1):
+    """(x, y, drop_ids, t_fm, t_mf, r_mf, eps_fm, eps_mf) for ``dmf_loss``: latents and
+    noises ~ N(0,1), labels uniform with a fraction ``cfg_prob`` replaced by the null
+    class, times logit-normal with the reference's defaults (loss.py:100-140), r <= t."""
+    g = torch.Generator().manual_seed(seed)
+    x, eps_fm, eps_mf = (torch.randn(batch, channels, input_size, input_size, generator=g) for _ in range(3))
+    y = torch.randint(0, num_classes, (batch,), generator=g)
+    drop_ids = torch.rand(batch, generator=g) < cfg_prob
+    y = torch.where(drop_ids, num_classes, y)
+    ln = lambda mean: torch.sigmoid(torch.randn(batch, 1, 1, 1, generator=g) + mean)
+    t_fm, a, b = ln(-0.4), ln(-0.2), ln(0.2)
+    return tuple(v.to(device) for v in (x, y, drop_ids, t_fm, torch.maximum(a, b), torch.minimum(a, b), eps_fm, eps_mf))
+
+
 def build_model(name: str, attn_func: str, device, qk_norm: bool = False, input_size: int = 32, dmf_depth=None, seed: int = 0,
-                block_ops: str = "torch"):
-    kw = {"attn_func": attn_func, "qk_norm": qk_norm, "input_size": input_size, "block_ops": block_ops}
+                block_ops: str = "torch", **extra):
+    """A DMFT (``"DMFT-*"``) or SiT (``"SiT-*"``) of the reference's size registry with truncated-normal weights."""
+    kw = {"attn_func": attn_func, "qk_norm": qk_norm, "input_size": input_size, "block_ops": block_ops, **extra}
     if dmf_depth is not None:
         kw["dmf_depth"] = dmf_depth
-    return DMFT_models[name](**kw).init_trunc_normal_(0.02, seed).to(device)
+    registry = SiT_models if name.startswith("SiT") else DMFT_models
+    return registry[name](**kw).init_trunc_normal_(0.02, seed).to(device)
 
 
 class GraphedStep:
@@ -81,7 +212,12 @@ class GraphedStep:
     pure function of its tensor arguments (and of module parameters, which are
     read in place at replay time); its outputs live in the graph's memory pool
     and are overwritten by the next call.  Capture happens on a side stream at
-    the default priority after ``warmup`` eager calls.
+    the default priority after ``warmup`` eager calls.  If ``fn`` runs a backward
+    pass, no autograd graph of an earlier step may be alive when the step is
+    captured (keep ``float(loss)`` or ``loss.detach()``, not ``loss``): a parameter's
+    gradient accumulator lives as long as any graph refers to it and stays bound to
+    the stream it was created on, so the captured backward would be sent to a stream
+    that is not capturing, which the runtime answers with a crash, not an error.
     """
 
     def __init__(self, fn, *example_inputs, warmup: int = 3):
@@ -122,7 +258,10 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     no-grad forward at batch 128 -- the call mode of the guidance branch
     (loss.py:64-69, a 2B batch) and of a sampler step (samplers.py:69-100) -- and
     (d) DMFT-XL/2 at 512px (1024 tokens) with qk-norm, forward+JVP, batch 16: the
-    caller of the headline attention shape.  Variants:
+    caller of the headline attention shape, (e) the whole DMF training step of
+    train_dmf.py on DMFT-XL/2 with model guidance (``dmf_train_step``: four model
+    calls, two of them no-grad on a 2B batch), batch 16, and (f) the flow-matching
+    training step of train_fm.py on SiT-XL/2 (``fm_train_step``), batch 32.  Variants:
     ``hip_fused_graph`` -- 'hip' attention + fused block glue, replayed as a HIP graph,
     ``hip_fused_fwad``  -- the same, launched eagerly with the forward-AD dual level opened directly,
     ``hip_fused``       -- the same, launched eagerly through ``torch.func.jvp`` (the reference's call),
@@ -133,23 +272,42 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     # (key, model, batch, dmf_depth, mode, latent size, qk_norm)
     all_cases = [("DMFT-B/2", "DMFT-B/2", 64, 8, "jvp", 32, False), ("DMFT-XL/2", "DMFT-XL/2", 32, 20, "train", 32, False),
                  ("DMFT-B/2 no-grad", "DMFT-B/2", 128, 8, "nograd", 32, False),
-                 ("DMFT-XL/2 512px qk-norm", "DMFT-XL/2", 16, 20, "jvp", 64, True)]
+                 ("DMFT-XL/2 512px qk-norm", "DMFT-XL/2", 16, 20, "jvp", 64, True),
+                 ("DMFT-XL/2 DMF loss step (mg)", "DMFT-XL/2", 16, 20, "dmf_loss", 32, False),
+                 ("SiT-XL/2 FM train step", "SiT-XL/2", 32, None, "fm", 32, False)]
     cases = [c for c in all_cases if only in (None, c[0])]
     all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused_fwad", "hip", "hip", False), ("hip_fused", "hip", "hip", False),
                     ("hip", "hip", "torch", False)]
     if compare_base:
         all_variants.append(("base", "base", "torch", False))
     variants = [v for v in all_variants if variants is None or v[0] in variants]
-    modes = {"jvp": "fwd+jvp", "train": "fwd+jvp+bwd", "nograd": "primal-only forward, no grad (guidance / sampler call)"}
+    modes = {"jvp": "fwd+jvp", "train": "fwd+jvp+bwd", "nograd": "primal-only forward, no grad (guidance / sampler call)",
+             "dmf_loss": "fwd(grad) + 2x guidance fwd (no grad, 2B) + fwd+jvp, then bwd", "fm": "fwd+bwd (no jvp)"}
     for key, name, batch, dmf_depth, mode, input_size, qk_norm in cases:
         row = {"batch": batch, "mode": modes[mode], "dtype": "bf16 autocast", "tokens": (input_size // 2) ** 2, "qk_norm": qk_norm}
-        data = synthetic_batch(batch, device, input_size=input_size)
+        if mode == "dmf_loss":
+            data = synthetic_loss_batch(batch, device, input_size=input_size)
+        elif mode == "fm":
+            x, y, _, t_fm, _, _, eps, _ = synthetic_loss_batch(batch, device, input_size=input_size)
+            data = (x, y, t_fm, eps)
+        else:
+            data = synthetic_batch(batch, device, input_size=input_size)
         for label, op, block_ops, graphed in variants:
-            if mode == "nograd" and label == "hip_fused_fwad":
+            if mode in ("nograd", "fm") and label == "hip_fused_fwad":
                 continue   # no JVP in this mode
-            model = build_model(name, op, device, qk_norm=qk_norm, input_size=input_size, dmf_depth=dmf_depth, block_ops=block_ops)
+            extra = {"use_logvar": True} if mode == "dmf_loss" else {}
+            model = build_model(name, op, device, qk_norm=qk_norm, input_size=input_size, dmf_depth=dmf_depth, block_ops=block_ops,
+                                **extra)
             functorch = label != "hip_fused_fwad"
-            if mode == "train":
+            if mode == "dmf_loss":
+                def step(*batch_tensors):
+                    model.zero_grad(set_to_none=True)
+                    return dmf_train_step(model, batch_tensors, functorch=functorch, g_type="mg", omega=0.5).detach()
+            elif mode == "fm":
+                def step(*batch_tensors):
+                    model.zero_grad(set_to_none=True)
+                    return fm_train_step(model, batch_tensors).detach()
+            elif mode == "train":
                 def step(*batch_tensors):
                     model.zero_grad(set_to_none=True)
                     return train_step(model, batch_tensors, functorch=functorch).detach()
@@ -166,7 +324,7 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
                     with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
                         return model(z, t, r, y)
             # the forward+JVP-only and no-grad passes run over frozen weights: cast them once, not per call
-            frozen = frozen_low_precision_params(model) if (mode != "train" and block_ops == "hip") else contextlib.nullcontext()
+            frozen = frozen_low_precision_params(model) if (mode in ("jvp", "nograd") and block_ops == "hip") else contextlib.nullcontext()
             with frozen:
                 run = GraphedStep(step, *data) if graphed else step
                 sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
