@@ -23,6 +23,7 @@ import torch.autograd.forward_ad as fwAD
 
 from .dmft import DMFT_models
 from .layers import frozen_low_precision_params
+from .samplers import euler_sampler
 from .sit import SiT_models
 
 
@@ -261,7 +262,10 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     caller of the headline attention shape, (e) the whole DMF training step of
     train_dmf.py on DMFT-XL/2 with model guidance (``dmf_train_step``: four model
     calls, two of them no-grad on a 2B batch), batch 16, and (f) the flow-matching
-    training step of train_fm.py on SiT-XL/2 (``fm_train_step``), batch 32.  Variants:
+    training step of train_fm.py on SiT-XL/2 (``fm_train_step``), batch 32, and (g)
+    generate.py's sampling loop: ``euler_sampler``, 4 steps with classifier-free
+    guidance 1.5 on t in [0, 0.8], DMFT-XL/2 cast to bf16, batch 64 (images/s counts
+    finished latents).  Variants:
     ``hip_fused_graph`` -- 'hip' attention + fused block glue, replayed as a HIP graph,
     ``hip_fused_fwad``  -- the same, launched eagerly with the forward-AD dual level opened directly,
     ``hip_fused``       -- the same, launched eagerly through ``torch.func.jvp`` (the reference's call),
@@ -274,7 +278,8 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
                  ("DMFT-B/2 no-grad", "DMFT-B/2", 128, 8, "nograd", 32, False),
                  ("DMFT-XL/2 512px qk-norm", "DMFT-XL/2", 16, 20, "jvp", 64, True),
                  ("DMFT-XL/2 DMF loss step (mg)", "DMFT-XL/2", 16, 20, "dmf_loss", 32, False),
-                 ("SiT-XL/2 FM train step", "SiT-XL/2", 32, None, "fm", 32, False)]
+                 ("SiT-XL/2 FM train step", "SiT-XL/2", 32, None, "fm", 32, False),
+                 ("DMFT-XL/2 4-step sampling cfg 1.5", "DMFT-XL/2", 64, 20, "sample", 32, False)]
     cases = [c for c in all_cases if only in (None, c[0])]
     all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused_fwad", "hip", "hip", False), ("hip_fused", "hip", "hip", False),
                     ("hip", "hip", "torch", False)]
@@ -282,24 +287,34 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
         all_variants.append(("base", "base", "torch", False))
     variants = [v for v in all_variants if variants is None or v[0] in variants]
     modes = {"jvp": "fwd+jvp", "train": "fwd+jvp+bwd", "nograd": "primal-only forward, no grad (guidance / sampler call)",
-             "dmf_loss": "fwd(grad) + 2x guidance fwd (no grad, 2B) + fwd+jvp, then bwd", "fm": "fwd+bwd (no jvp)"}
+             "dmf_loss": "fwd(grad) + 2x guidance fwd (no grad, 2B) + fwd+jvp, then bwd", "fm": "fwd+bwd (no jvp)",
+             "sample": "4 no-grad forwards (3 of them on a 2B batch) + fp64 Euler updates"}
     for key, name, batch, dmf_depth, mode, input_size, qk_norm in cases:
-        row = {"batch": batch, "mode": modes[mode], "dtype": "bf16 autocast", "tokens": (input_size // 2) ** 2, "qk_norm": qk_norm}
+        row = {"batch": batch, "mode": modes[mode], "dtype": "bf16 model" if mode == "sample" else "bf16 autocast",
+               "tokens": (input_size // 2) ** 2, "qk_norm": qk_norm}
         if mode == "dmf_loss":
             data = synthetic_loss_batch(batch, device, input_size=input_size)
         elif mode == "fm":
             x, y, _, t_fm, _, _, eps, _ = synthetic_loss_batch(batch, device, input_size=input_size)
             data = (x, y, t_fm, eps)
+        elif mode == "sample":
+            z, _, _, y, _ = synthetic_batch(batch, device, input_size=input_size)
+            data = (z.to(torch.bfloat16), y)
         else:
             data = synthetic_batch(batch, device, input_size=input_size)
         for label, op, block_ops, graphed in variants:
-            if mode in ("nograd", "fm") and label == "hip_fused_fwad":
+            if mode in ("nograd", "fm", "sample") and label == "hip_fused_fwad":
                 continue   # no JVP in this mode
             extra = {"use_logvar": True} if mode == "dmf_loss" else {}
             model = build_model(name, op, device, qk_norm=qk_norm, input_size=input_size, dmf_depth=dmf_depth, block_ops=block_ops,
                                 **extra)
             functorch = label != "hip_fused_fwad"
-            if mode == "dmf_loss":
+            if mode == "sample":
+                model = model.to(torch.bfloat16).eval().requires_grad_(False)     # generate.py:84-85
+
+                def step(z, y):
+                    return euler_sampler(model, z, y, num_steps=4, cfg_scale=1.5, g_min=0.0, g_max=0.8)
+            elif mode == "dmf_loss":
                 def step(*batch_tensors):
                     model.zero_grad(set_to_none=True)
                     return dmf_train_step(model, batch_tensors, functorch=functorch, g_type="mg", omega=0.5).detach()

@@ -20,6 +20,8 @@ def _dmft(attn_func, **kw):
     cfg = dict(input_size=8, patch_size=2, hidden_size=64, depth=3, num_heads=4, dmf_depth=2, attn_func=attn_func, use_logvar=True)
     cfg.update(kw)
     m = DMFT(**cfg).init_trunc_normal_(0.02, seed=1)
+    if not m.use_logvar:
+        return m
     with torch.no_grad():   # a log-variance head that is not identically zero
         m.logvar_linear.weight.copy_(0.05 * torch.randn(m.logvar_linear.weight.shape, generator=torch.Generator().manual_seed(3)))
         m.logvar_linear.bias.fill_(0.1)
@@ -269,3 +271,86 @@ def test_sit_projector_features_fused_vs_torch_under_jvp():
     (o2, z2), (to2, tz2) = f(m_ref)
     for a, b in ((o1, o2), (z1[0], z2[0]), (to1, to2), (tz1[0], tz2[0])):
         assert ao.rel_l2(a, b) <= 2e-4
+
+
+# ---- sampling loop (dmf_amd/samplers.py) ---------------------------------------------------------------------------
+
+def test_get_tsteps_closed_form():
+    from dmf_amd.samplers import get_tsteps
+    t = get_tsteps(4)
+    assert t.dtype == torch.float64 and t.tolist() == [1.0, 0.75, 0.5, 0.25, 0.0]
+    s = get_tsteps(4, shift=3.0)
+    assert torch.allclose(s, 3 * t / (1 + 2 * t)) and s[0] == 1.0 and s[-1] == 0.0 and float(s[2]) == 0.75
+
+
+class _Field(torch.nn.Module):
+    """d(x, t, r, y) = a(y) * x + t - 2 r with a = 1 for real labels and 3 for the null class; records (n, t, r)."""
+
+    def __init__(self):
+        super().__init__()
+        self.calls = []
+
+    def forward(self, x, t, r, y):
+        assert not torch.is_grad_enabled()
+        self.calls.append((x.shape[0], float(t[0]), float(r[0]), x.dtype))
+        a = torch.where(y == 1000, 3.0, 1.0).view(-1, 1, 1, 1).to(x.dtype)
+        return a * x + (t - 2 * r).view(-1, 1, 1, 1)
+
+
+def test_euler_sampler_known_answers():
+    from dmf_amd.samplers import euler_sampler
+    x0 = torch.randn(3, 4, 2, 2, generator=torch.Generator().manual_seed(5))
+    y = torch.tensor([1, 2, 3])
+    f = _Field()
+    out = euler_sampler(f, x0, y, num_steps=2)
+    # two explicit Euler steps of x' = x + t - 2 r from t = 1 to 0.5 to 0, by hand in fp64 (r = next time)
+    x = x0.double()
+    x = x + (0.5 - 1.0) * (x + 1.0 - 2 * 0.5)
+    x = x + (0.0 - 0.5) * (x + 0.5 - 0.0)
+    assert out.dtype == torch.float64 and torch.allclose(out, x, atol=1e-6)
+    assert [(n, t, r) for n, t, r, _ in f.calls] == [(3, 1.0, 0.5), (3, 0.5, 0.0)] and f.calls[0][3] == torch.float32
+    # guidance: doubled batch inside the window only; d = d_uncond + w (d_cond - d_uncond)
+    f = _Field()
+    out = euler_sampler(f, x0, y, num_steps=2, cfg_scale=2.0, g_min=0.0, g_max=0.75)
+    x = x0.double()
+    x = x + (0.5 - 1.0) * (x + 1.0 - 1.0)                                    # t = 1 is outside the window: plain step
+    d_c, d_u = x + 0.5, 3 * x + 0.5
+    x = x + (0.0 - 0.5) * (d_u + 2.0 * (d_c - d_u))
+    assert torch.allclose(out, x, atol=1e-6) and [c[0] for c in f.calls] == [3, 6]
+    # the model is called in the dtype of the latents, the state is carried in fp64
+    f = _Field()
+    euler_sampler(f, x0.bfloat16(), y, num_steps=1)
+    assert f.calls[0][3] == torch.bfloat16
+
+
+@pytest.mark.gpu
+def test_euler_sampler_bf16_model_fused_vs_base():
+    """generate.py's setting: the model cast to bf16 (parameters included), 4 steps
+    with classifier-free guidance; 'hip' attention + fused block glue against the
+    naive attention and the reference's expressions on the same weights, and the
+    model call replayed from a HIP graph against the eager call."""
+    from dmf_amd.samplers import euler_sampler
+    dev = "cuda:0"
+    kw = dict(input_size=32, hidden_size=288, depth=4, num_heads=4, dmf_depth=3, qk_norm=True, use_logvar=False)
+    m_ref = _dmft("base", **kw)
+    m = _dmft("hip", block_ops="hip", **kw)
+    m.load_state_dict(m_ref.state_dict())
+    m_ref, m = m_ref.to(dev, torch.bfloat16).eval(), m.to(dev, torch.bfloat16).eval()
+    g = torch.Generator().manual_seed(11)
+    z = torch.randn(8, 4, 32, 32, generator=g).to(dev, torch.bfloat16)
+    y = torch.randint(0, 1000, (8,), generator=g).to(dev)
+    args = dict(num_steps=4, cfg_scale=1.5, g_min=0.0, g_max=0.8, shift=1.5)
+    ref = euler_sampler(m_ref, z, y, **args)
+    out = euler_sampler(m, z, y, **args)
+    assert out.dtype == torch.float64 and ao.rel_l2(out, ref) <= 3e-2
+    graphs = {}
+
+    def call(x, t, r, yy):
+        n = x.shape[0]
+        if n not in graphs:
+            with torch.no_grad():
+                graphs[n] = harness.GraphedStep(lambda *a: m(*a), x, t, r, yy)
+        return graphs[n](x, t, r, yy)
+
+    out_g = euler_sampler(m, z, y, model_call=call, **args)
+    assert sorted(graphs) == [8, 16] and ao.rel_l2(out_g, out) <= 1e-6
