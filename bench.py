@@ -42,6 +42,14 @@ WORKLOADS = {
 }
 
 
+_T0 = time.perf_counter()
+
+
+def progress(text):
+    """One line per finished measurement on stderr (stdout carries only the final JSON line)."""
+    print(f"[bench {time.perf_counter() - _T0:6.1f}s] {text}", file=sys.stderr, flush=True)
+
+
 def make_inputs(name, device, dtype, seed):
     import torch
     from dmf_amd.layers import RMSNorm
@@ -282,6 +290,7 @@ def main():
     flops = attn_flops(B, H, N, D, "fwd_jvp")
     tflops = flops / (ms * 1e-3) / 1e12
     ms_median, ms_min = per_launch_stats(lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale))
+    progress(f"{name} attention fwd+JVP: {ms:.4f} ms/step, {tflops:.1f} TFLOP/s")
     result = {
         "metric": "attn_fwd_jvp_tflops", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
@@ -313,17 +322,21 @@ def main():
                 row[kind] = {"ms": t_ms, "tflops": fl / t_ms / 1e9, "pct_bf16_mfma_peak": 100 * fl / t_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
                              "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS}
             extra[wname] = row
+            progress(f"{wname}: fwd_jvp / fwd / bwd = " + " / ".join(f"{row[kd]['ms']:.4f}" for kd in ("fwd_jvp", "fwd", "bwd")) + " ms")
             del ins
         extra["device_probes"] = device_probes()
+        progress("device probes done")
         extra["block_kernels"] = block_kernel_rows(dev)
+        progress("block kernels done")
         try:
             from dmf_amd import harness
-            extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10))
+            extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10), log=progress)
         except ImportError:
             pass
         result["extra"] = extra
 
     if not args.no_cpu:
+        progress("CPU baseline (bounded sample) ...")
         result["cpu_baseline"] = cpu_baseline(name)
         if not args.no_extra:
             result["extra"]["cpu_config1"] = cpu_baseline_config1()

@@ -191,7 +191,7 @@ ENOKERNEL = -8   # DMF_ATTN_ENOKERNEL
 
 def fwd_qnorm(q, k, v, tq, tk, tv, q_gain, eps: float, scale: float, need_lse: bool = True):
     """Forward (+ JVP when ``tq`` is given) with the per-head RMS norm of q (gain
-    ``q_gain``, fp32 (D)) applied inside the attention kernel.  Returns (o, to, lse)
+    ``q_gain``, (D), fp32 or exactly representable in it) applied inside the attention kernel.  Returns (o, to, lse)
     (``to`` None without tangents), or None when no kernel implements the variant for
     this shape / dtype -- the caller then normalises q itself."""
     jvp = tq is not None
@@ -204,8 +204,10 @@ def fwd_qnorm(q, k, v, tq, tk, tv, q_gain, eps: float, scale: float, need_lse: b
     gain = _raw(q_gain)
     if gain.dim() != 1 or gain.shape[0] != q.shape[-1] or gain.device != q.device:
         raise ValueError("fwd_qnorm: q_gain must be a (D) tensor on the device of q")
-    gain = _raw(gain.contiguous())
-    if q.dtype != torch.bfloat16 or gain.dtype != torch.float32 or gain.data_ptr() % 16:
+    if q.dtype != torch.bfloat16:
+        return None
+    gain = _raw(gain.float().contiguous())   # exact for a bf16 gain (a model cast to bf16 as a whole)
+    if gain.data_ptr() % 16:
         return None
     B, Lq, H, D = q.shape
     Lkv = k.shape[1]

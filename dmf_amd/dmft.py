@@ -82,13 +82,18 @@ def trunc_normal_init_(model: nn.Module, std: float = 0.02, seed: int = 0) -> nn
     """Benchmark initialisation: every weight matrix / embedding ~ truncated
     N(0, std) (cut at 2 std), biases zero.  With the reference's zero-gate
     initialisation attention contributes nothing to the output, so timing and
-    parity runs use this instead."""
-    g = torch.Generator().manual_seed(seed)
+    parity runs use this instead.  Values are drawn on the device the parameters live
+    on (a model built on the GPU is initialised there, in a fraction of the time), so
+    the same seed gives different weights on different device types."""
+    gens = {}
     for name, prm in model.named_parameters():
         if name == "pos_embed":
             continue
         if prm.dim() >= 2:
-            w = torch.empty(prm.shape, dtype=torch.float32)
+            g = gens.get(prm.device)
+            if g is None:
+                g = gens[prm.device] = torch.Generator(device=prm.device).manual_seed(seed)
+            w = torch.empty(prm.shape, dtype=torch.float32, device=prm.device)
             nn.init.trunc_normal_(w, std=std, a=-2 * std, b=2 * std, generator=g)
             prm.data.copy_(w)
         elif name.endswith("bias"):

@@ -195,12 +195,15 @@ def synthetic_loss_batch(batch: int, device, seed: int = 3, input_size: int = 32
 
 def build_model(name: str, attn_func: str, device, qk_norm: bool = False, input_size: int = 32, dmf_depth=None, seed: int = 0,
                 block_ops: str = "torch", **extra):
-    """A DMFT (``"DMFT-*"``) or SiT (``"SiT-*"``) of the reference's size registry with truncated-normal weights."""
+    """A DMFT (``"DMFT-*"``) or SiT (``"SiT-*"``) of the reference's size registry with truncated-normal weights,
+    constructed and initialised directly on ``device``."""
     kw = {"attn_func": attn_func, "qk_norm": qk_norm, "input_size": input_size, "block_ops": block_ops, **extra}
     if dmf_depth is not None:
         kw["dmf_depth"] = dmf_depth
     registry = SiT_models if name.startswith("SiT") else DMFT_models
-    return registry[name](**kw).init_trunc_normal_(0.02, seed).to(device)
+    with torch.device(device):
+        model = registry[name](**kw)
+    return model.init_trunc_normal_(0.02, seed)
 
 
 class GraphedStep:
@@ -253,7 +256,7 @@ def _time(fn, steps: int, warmup: int = 2) -> float:
     return (time.perf_counter() - t0) / steps
 
 
-def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=None, variants=None) -> dict:
+def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=None, variants=None, log=None) -> dict:
     """images/s for (a) DMFT-B/2 256px forward+JVP, batch 64, bf16 autocast,
     (b) DMFT-XL/2 256px forward+JVP+backward, batch 32, and (c) DMFT-B/2 primal-only
     no-grad forward at batch 128 -- the call mode of the guidance branch
@@ -271,7 +274,8 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     ``hip_fused``       -- the same, launched eagerly through ``torch.func.jvp`` (the reference's call),
     ``hip``             -- 'hip' attention inside the reference's tensor expressions,
     ``base``            -- naive attention (the reference's own CPU-runnable operator).
-    ``only`` / ``variants`` restrict the model / the variants that are run."""
+    ``only`` / ``variants`` restrict the model / the variants that are run; ``log(text)``
+    is called after every measurement."""
     out = {}
     # (key, model, batch, dmf_depth, mode, latent size, qk_norm)
     all_cases = [("DMFT-B/2", "DMFT-B/2", 64, 8, "jvp", 32, False), ("DMFT-XL/2", "DMFT-XL/2", 32, 20, "train", 32, False),
@@ -345,6 +349,8 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
                 sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
             row[f"{label}_ms_per_step"] = sec * 1e3
             row[f"{label}_images_per_s"] = batch / sec
+            if log is not None:
+                log(f"{key} [{label}]: {sec * 1e3:.2f} ms/step, {batch / sec:.1f} images/s")
             del model, run, step
             torch.cuda.empty_cache()
         out[key] = row
