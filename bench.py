@@ -251,9 +251,9 @@ def main():
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch one plain 1 GiB device copy (reads 1 GiB, writes 1 GiB): the known-size kernel "
                          "that HBM traffic counters are scaled by when this command runs under rocprofv3 --pmc")
-    ap.add_argument("--dmft-graph", choices=["DMFT-B/2", "DMFT-XL/2"], default=None,
-                    help="profiling aid: run only the HIP-graph replay of the fused DMFT step (B/2: forward+JVP, batch 64; "
-                         "XL/2: forward+JVP+backward, batch 32) for --steps replays and print its images/s")
+    ap.add_argument("--dmft-graph", default=None, metavar="CASE",
+                    help="profiling aid: run only the HIP-graph replay of one fused end-to-end case of extra.dmft (its key, e.g. "
+                         "'DMFT-B/2', 'DMFT-XL/2', 'SiT-XL/2 FM train step') for --steps replays and print its images/s")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the attention units (b, h) are independent and shard "
@@ -268,11 +268,14 @@ def main():
     dev, dtype = "cuda:0", torch.bfloat16
     if args.dmft_graph:
         from dmf_amd import harness
-        row = harness.bench_dmft(steps=max(1, args.steps // 4), only=args.dmft_graph, variants=("hip_fused_graph",))[args.dmft_graph]
+        rows = harness.bench_dmft(steps=max(1, args.steps // 4), only=args.dmft_graph, variants=("hip_fused_graph",))
+        if args.dmft_graph not in rows:
+            sys.exit(f"bench.py: unknown --dmft-graph case {args.dmft_graph!r}")
+        row = rows[args.dmft_graph]
         print(json.dumps({"metric": "dmft_images_per_s", "value": row["hip_fused_graph_images_per_s"], "unit": "images/s",
                           "n_gpus": 1, "steps": args.steps, "ms_per_step": row["hip_fused_graph_ms_per_step"],
-                          "config": {"workload": f"{args.dmft_graph} 256px {row['mode']} batch {row['batch']} bf16 autocast, "
-                                                 "hip attention + fused block glue, HIP-graph replay"}}))
+                          "config": {"workload": f"{args.dmft_graph}: {row['tokens']} tokens, {row['mode']}, batch {row['batch']}, "
+                                                 f"{row['dtype']}, hip attention + fused block glue, HIP-graph replay"}}))
         return
     name = args.workload
     B, H, N, D, _ = WORKLOADS[name]
