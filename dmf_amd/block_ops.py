@@ -10,6 +10,7 @@ attention operator in the reference's block (models/layers.py):
 * ``rms_norm(x, gain)``             = ``RMSNorm.forward``                        (:33-42, :148)
 * ``silu(x)``                       = ``nn.SiLU()`` of the adaLN branch          (:185-188, :211-214)
 * ``dual_linear(x, weight, bias)``  = ``nn.Linear`` (:131,137,161-165,...) -- library GEMMs, see ``DualLinearFunc``
+* ``linear_gelu_tanh(x, weight, bias)`` = ``act(fc1(x))`` of the MLP (:166) -- GELU in the GEMM epilogue when nothing is differentiated
 
 Each follows the protocol of the attention operator (flash_attention_hip_jvp):
 a wrapper unpacks forward-AD duals, one ``torch.autograd.Function`` call pushes
@@ -267,6 +268,22 @@ def dual_linear(x, weight, bias=None, w_lp=None, b_lp=None):
     (xp,), (tx,), dual = _unpack(x)
     y, ty, _ = _lib.run_function(DualLinearFunc, xp, tx, weight, bias, w_lp, b_lp)
     return fwAD.make_dual(y, ty) if dual else y
+
+
+def linear_gelu_tanh(x, weight, bias, w_lp=None, b_lp=None):
+    """``gelu_tanh(F.linear(x, weight, bias))`` -- the first half of the MLP
+    (reference models/layers.py:161-166).  Without gradients and without a tangent
+    the activation rides in the GEMM's epilogue (one library call, the pre-activation
+    never reaches HBM); otherwise the pre-activation is needed for the tangent and for
+    the backward pass and this is ``dual_linear`` followed by ``gelu_tanh``."""
+    if torch.is_grad_enabled() or bias is None or not x.is_cuda or fwAD.unpack_dual(x).tangent is not None:
+        return gelu_tanh(dual_linear(x, weight, bias, w_lp, b_lp))
+    dt = _autocast_dtype(x)
+    cached = w_lp is not None and w_lp.dtype == dt
+    w = w_lp if cached else weight.to(dt)
+    b = b_lp if cached and b_lp is not None else bias.to(dt)
+    x2 = _lib._raw(x).reshape(-1, x.shape[-1]).to(dt)
+    return torch._addmm_activation(b, x2, _lib._raw(w).t(), use_gelu=True).reshape(*x.shape[:-1], w.shape[0])
 
 
 def _autocast_dtype(x: torch.Tensor):

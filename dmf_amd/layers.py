@@ -208,6 +208,8 @@ class Mlp(nn.Module):
         self.fc2 = Linear(hidden_features, in_features, block_ops=block_ops)
 
     def forward(self, x: Tensor) -> Tensor:
+        if self.fc1.fused:
+            return self.fc2(fused.linear_gelu_tanh(x, self.fc1.weight, self.fc1.bias, self.fc1.lp_weight, self.fc1.lp_bias))
         return self.fc2(self.act(self.fc1(x)))
 
 

@@ -337,3 +337,33 @@ def test_golden_vectors():
     gx, gg = _lib.rmsnorm_bwd(g("rms.gy"), g("rms.x"), g("rms.gain"))
     for got, key in ((y, "rms.y"), (ty, "rms.ty"), (gx, "rms.gx"), (gg, "rms.ggain")):
         _close(got, ref(key), 1e-5, key)
+
+
+@pytest.mark.parametrize("mode", ["bf16", "autocast", "fp32"])
+def test_linear_gelu_tanh_epilogue_path(mode):
+    """``linear_gelu_tanh`` without gradients (GELU in the GEMM epilogue) against the
+    oracle's tanh-GELU of an fp32 linear, and against the two-kernel path that is
+    taken as soon as a gradient or a tangent is involved."""
+    g = torch.Generator().manual_seed(41)
+    x = torch.randn(3, 50, 96, generator=g).to(DEV)
+    w = (0.1 * torch.randn(384, 96, generator=g)).to(DEV)
+    b = (0.5 * torch.randn(384, generator=g)).to(DEV)
+    if mode == "bf16":
+        x, w, b = x.bfloat16(), w.bfloat16(), b.bfloat16()
+    ref = bo.gelu_tanh(torch.nn.functional.linear(x.float().cpu(), w.float().cpu(), b.float().cpu()))
+    tol = 1e-5 if mode == "fp32" else 8e-3
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=mode == "autocast"):
+        with torch.no_grad():
+            y = block_ops.linear_gelu_tanh(x, w, b)
+            y_lp = block_ops.linear_gelu_tanh(x, w, b, w.bfloat16(), b.bfloat16())      # pre-cast copies
+        y2 = block_ops.linear_gelu_tanh(x, w.requires_grad_(), b)                          # grad mode: two kernels
+        t = torch.randn(x.shape, generator=g).to(x)
+        yd, tyd = torch.func.jvp(lambda a: block_ops.linear_gelu_tanh(a, w.detach(), b), (x,), (t,))
+    assert y.shape == (3, 50, 384) and y.dtype == (torch.float32 if mode == "fp32" else torch.bfloat16)
+    for got in (y, y_lp, y2, yd):
+        assert ao.rel_l2(got.float().cpu(), ref) <= tol
+    _, t_ref = bo.jvp(lambda a: bo.gelu_tanh(torch.nn.functional.linear(a, w.detach().float().cpu(), b.float().cpu())),
+                      (x.float().cpu(),), (t.float().cpu(),))
+    assert ao.rel_l2(tyd.float().cpu(), t_ref) <= tol
+    y2.float().sum().backward()
+    assert w.grad is not None and float(w.grad.abs().max()) > 0
