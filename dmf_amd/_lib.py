@@ -13,6 +13,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 import torch
 from torch._C import _functorch
 from torch._functorch.pyfunctorch import retrieve_all_functorch_interpreters as _interpreters
+from torch._functorch.pyfunctorch import temporarily_pop_interpreter_stack as _pop_interpreter
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdmf_attn.so")
@@ -87,17 +88,39 @@ def _raw(t):
     return t
 
 
+# Call custom Functions below a single torch.func.jvp level instead of through it (module switch for A/B timing and tests).
+BASE_LEVEL_UNDER_JVP = True
+
+
 def run_function(fn_cls, *args):
-    """``fn_cls.apply(*args)`` -- or, when nothing needs a gradient and no functorch
-    transform other than ``jvp`` is active, ``fn_cls.forward(*args)`` directly.  The
-    operators of this package unpack forward-AD duals themselves, so the only thing
-    ``apply`` adds then is the (considerable) per-call cost of building an autograd
-    node through functorch's custom-Function dispatch."""
+    """``fn_cls.apply(*args)`` without functorch's custom-Function dispatch where that
+    is sound.  The operators of this package unpack forward-AD duals themselves and
+    pass primals and tangents as separate arguments, so inside ``torch.func.jvp`` the
+    dispatch adds nothing but its (considerable, ~0.2-0.4 ms) per-call cost:
+
+    * nothing needs a gradient and only ``jvp`` levels are active: ``fn_cls.forward``
+      is called directly;
+    * a gradient is needed and exactly one ``jvp`` level is active: the arguments are
+      unwrapped, ``apply`` runs below the level like the ordinary autograd node it is,
+      and the outputs are wrapped for the level again (what functorch does for every
+      built-in operator);
+    * otherwise (no transform, nested levels, ``vmap`` / ``grad``): plain ``apply``."""
+    stack = _interpreters()
+    if not stack:
+        return fn_cls.apply(*args)
     # (inside a functorch level the wrapper tensors do not report requires_grad; the wrapped values do)
     needs_grad = torch.is_grad_enabled() and any(isinstance(a, torch.Tensor) and (a.requires_grad or _raw(a).requires_grad)
                                                  for a in args)
-    if not needs_grad and all(i.key() == _functorch.TransformType.Jvp for i in _interpreters()):
+    only_jvp = all(i.key() == _functorch.TransformType.Jvp for i in stack)
+    if not needs_grad and only_jvp:
         return fn_cls.forward(*args)
+    if BASE_LEVEL_UNDER_JVP and only_jvp and len(stack) == 1:
+        level = stack[0].level()
+        raw_args = [_raw(a) if isinstance(a, torch.Tensor) else a for a in args]
+        with _pop_interpreter():
+            outs = fn_cls.apply(*raw_args)
+        wrap = lambda o: _functorch._wrap_for_grad(o, level) if isinstance(o, torch.Tensor) else o
+        return tuple(wrap(o) for o in outs) if isinstance(outs, tuple) else wrap(outs)
     return fn_cls.apply(*args)
 
 
