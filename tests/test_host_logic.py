@@ -215,3 +215,68 @@ def test_block_abi_validation_codes_without_launch():
     assert lib.dmf_block_workspace_floats(1, 2, 33, 64) == 2 * 3 * 64
     assert lib.dmf_block_workspace_floats(2, 1, 1, 72) == 1024 * 72
     assert lib.dmf_block_workspace_floats(9, 1, 1, 72) == 0
+
+
+def test_run_function_below_a_single_jvp_level_matches_functorch_dispatch(monkeypatch):
+    """``_lib.run_function`` with a gradient needed inside one ``torch.func.jvp`` level:
+    running the autograd node below the level gives the values and gradients of
+    functorch's own custom-Function dispatch; other transforms keep using ``apply``."""
+    import torch.autograd.forward_ad as fwAD
+
+    class Scale(torch.autograd.Function):
+        """(x, tx, w) -> (x w, tx w), gradient through the primal output only."""
+        calls = []
+
+        @staticmethod
+        def forward(x, tx, w):
+            return x * w, (None if tx is None else tx * w)
+
+        @staticmethod
+        def setup_context(ctx, inputs, outputs):
+            ctx.save_for_backward(inputs[0], inputs[2])
+            ctx.set_materialize_grads(False)
+            Scale.calls.append(_lib._functorch.is_functorch_wrapped_tensor(inputs[0]))
+
+        @staticmethod
+        def backward(ctx, gy, gty):
+            x, w = ctx.saved_tensors
+            return gy * w, None, (gy * x).sum(0)
+
+    def op(x, w):
+        p, t = fwAD.unpack_dual(x)
+        y, ty = _lib.run_function(Scale, p, t, w)
+        return y if t is None else fwAD.make_dual(y, ty)
+
+    g = torch.Generator().manual_seed(9)
+    w = torch.randn(8, generator=g).requires_grad_()
+    x, v = torch.randn(4, 8, generator=g), torch.randn(4, 8, generator=g)
+    f = lambda a: op(torch.tanh(op(a, w)), w)
+    results = []
+    for flag in (True, False):
+        monkeypatch.setattr(_lib, "BASE_LEVEL_UNDER_JVP", flag)
+        Scale.calls.clear()
+        w.grad = None
+        y, ty = torch.func.jvp(f, (x,), (v,))
+        ((y - (0.5 * ty).detach()) ** 2).mean().backward()
+        results.append((y.detach(), ty.detach(), w.grad.clone()))
+        # below the level the node sees raw tensors, once per call; functorch's dispatch hands it wrapped ones as well
+        assert Scale.calls == [False, False] if flag else any(Scale.calls)
+    for a, b in zip(*results):
+        assert torch.allclose(a, b, rtol=1e-6, atol=1e-7)
+    # tangent against central differences, gradient against plain autograd of the same expression
+    h = 1e-3
+    fd = (f(x + h * v) - f(x - h * v)) / (2 * h)
+    assert torch.allclose(results[0][1], fd.detach(), atol=1e-3)
+    w.grad = None
+    yy = f(x)
+    ((yy - (0.5 * results[0][1])) ** 2).mean().backward()
+    assert torch.allclose(results[0][2], w.grad, rtol=1e-5, atol=1e-6)
+    # no gradient needed: forward is called directly (no autograd node at all)
+    monkeypatch.setattr(_lib, "BASE_LEVEL_UNDER_JVP", True)
+    Scale.calls.clear()
+    torch.func.jvp(lambda a: op(a, w.detach()), (x,), (v,))
+    assert Scale.calls == []
+    # a grad transform is not a jvp level: plain apply
+    Scale.calls.clear()
+    gx = torch.func.grad(lambda a: op(a, w.detach()).sum())(x)
+    assert torch.allclose(gx, w.detach().expand_as(x)) and any(Scale.calls)
