@@ -6,6 +6,7 @@ library raises ``RuntimeError`` at the first call.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
@@ -88,6 +89,15 @@ def _raw(t):
     return t
 
 
+def _apply(fn_cls, args):
+    """``fn_cls.apply(*args)`` minus what ``torch.autograd.Function.apply`` does in Python
+    before handing over to the C++ node constructor: binding the arguments against
+    ``inspect.signature(forward)`` (~40 us per call; every caller in this package passes
+    all arguments positionally) and the functorch check (the caller has made sure that
+    no transform is active)."""
+    return super(torch.autograd.Function, fn_cls).apply(*args)
+
+
 # Call custom Functions below a single torch.func.jvp level instead of through it (module switch for A/B timing and tests).
 BASE_LEVEL_UNDER_JVP = True
 
@@ -107,7 +117,7 @@ def run_function(fn_cls, *args):
     * otherwise (no transform, nested levels, ``vmap`` / ``grad``): plain ``apply``."""
     stack = _interpreters()
     if not stack:
-        return fn_cls.apply(*args)
+        return _apply(fn_cls, args)
     # (inside a functorch level the wrapper tensors do not report requires_grad; the wrapped values do)
     needs_grad = torch.is_grad_enabled() and any(isinstance(a, torch.Tensor) and (a.requires_grad or _raw(a).requires_grad)
                                                  for a in args)
@@ -118,7 +128,7 @@ def run_function(fn_cls, *args):
         level = stack[0].level()
         raw_args = [_raw(a) if isinstance(a, torch.Tensor) else a for a in args]
         with _pop_interpreter():
-            outs = fn_cls.apply(*raw_args)
+            outs = _apply(fn_cls, raw_args)
         wrap = lambda o: _functorch._wrap_for_grad(o, level) if isinstance(o, torch.Tensor) else o
         return tuple(wrap(o) for o in outs) if isinstance(outs, tuple) else wrap(outs)
     return fn_cls.apply(*args)
@@ -136,6 +146,14 @@ def side_stream(device) -> torch.cuda.Stream:
     if key not in _SIDE_STREAMS:
         _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
     return _SIDE_STREAMS[key]
+
+
+_NO_GUARD = contextlib.nullcontext()
+
+
+def _on(device):
+    """Context that makes ``device`` current for the launch -- nothing at all when it already is."""
+    return _NO_GUARD if device.index == torch.cuda.current_device() else torch.cuda.device(device)
 
 
 def _empty(shape, dtype, device) -> torch.Tensor:
@@ -183,7 +201,7 @@ def fwd_jvp(q, k, v, tq, tk, tv, scale: float, need_dlse: bool = False):
     to = _empty((B, Lq, H, D), q.dtype, q.device)
     lse = _empty((B, H, Lq), torch.float32, q.device)
     dlse = _empty((B, H, Lq), torch.float32, q.device) if need_dlse else None
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = load().dmf_attn_fwd_jvp(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(),
             o.data_ptr(), to.data_ptr(), lse.data_ptr(), dlse.data_ptr() if need_dlse else None,
@@ -201,7 +219,7 @@ def fwd(q, k, v, scale: float, need_lse: bool = True):
     Lkv = k.shape[1]
     o = _empty((B, Lq, H, D), q.dtype, q.device)
     lse = _empty((B, H, Lq), torch.float32, q.device) if need_lse else None
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = load().dmf_attn_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if need_lse else None,
             _strides(q, k, v, o), B, H, Lq, Lkv, D, float(scale), _dtype_code(q), _stream(q))
@@ -238,7 +256,7 @@ def fwd_qnorm(q, k, v, tq, tk, tv, q_gain, eps: float, scale: float, need_lse: b
     to = _empty((B, Lq, H, D), q.dtype, q.device) if jvp else None
     lse = _empty((B, H, Lq), torch.float32, q.device) if (need_lse or jvp) else None
     z = q   # stands in for absent tangents in the stride table (ignored by the library)
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = load().dmf_attn_fwd_qnorm(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), _ptr(tq), _ptr(tk), _ptr(tv), gain.data_ptr(), float(eps),
             o.data_ptr(), _ptr(to), _ptr(lse), None,
@@ -270,7 +288,7 @@ def bwd(dout, q, k, v, o, lse, scale: float, out=None):
         if dq.shape != q.shape or dk.shape != k.shape or dv.shape != v.shape:
             raise ValueError("bwd: `out` tensors must have the shapes of q, k, v")
     delta = _empty((B, H, Lq), torch.float32, q.device)
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = load().dmf_attn_bwd(
             dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(),
@@ -338,7 +356,7 @@ def ln_modulate_fwd(x, shift, scale, tx=None, tshift=None, tscale=None, eps: flo
     out_dtype = out_dtype or x.dtype
     y = _empty((B, L, C), out_dtype, x.device)
     ty = _empty((B, L, C), out_dtype, x.device) if jvp else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_ln_modulate_fwd(
             x.data_ptr(), _ptr(tx), shift.data_ptr(), scale.data_ptr(), _ptr(tshift), _ptr(tscale), y.data_ptr(), _ptr(ty),
             (c_int64 * 4)(s0, s1, s2, s3), B, L, C, float(eps), _dtype_code(x), _dtype_code(shift), _dtype_code(y), _stream(x))
@@ -357,7 +375,7 @@ def ln_modulate_bwd(gy, x, scale, eps: float = 1e-6, gres=None):
     gshift = _empty((B, C), scale.dtype, x.device)
     gscale = _empty((B, C), scale.dtype, x.device)
     ws = _workspace(0, B, L, C, x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_ln_modulate_bwd(
             gy.data_ptr(), x.data_ptr(), scale.data_ptr(), _ptr(gres), gx.data_ptr(), gshift.data_ptr(), gscale.data_ptr(),
             ws.data_ptr(), ss, B, L, C, float(eps), _dtype_code(x), _dtype_code(scale), _dtype_code(gy), _stream(x))
@@ -377,7 +395,7 @@ def gate_residual_fwd(x, gate, h, tx=None, tgate=None, th=None, jvp=False):
     (gate, g0), (tgate, g1) = _mod(gate, B, C), _mod(tgate, B, C)
     y = _empty((B, L, C), x.dtype, x.device)
     ty = _empty((B, L, C), x.dtype, x.device) if jvp else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_gate_residual_fwd(
             x.data_ptr(), _ptr(tx), gate.data_ptr(), _ptr(tgate), h.data_ptr(), _ptr(th), y.data_ptr(), _ptr(ty),
             (c_int64 * 2)(g0, g1), B, L, C, _dtype_code(x), _dtype_code(gate), _dtype_code(h), _stream(x))
@@ -393,7 +411,7 @@ def gate_residual_bwd(gy, gate, h):
     gh = _empty((B, L, C), h.dtype, h.device)
     ggate = _empty((B, C), gate.dtype, h.device)
     ws = _workspace(1, B, L, C, h.device)
-    with torch.cuda.device(h.device):
+    with _on(h.device):
         rc = load().dmf_gate_residual_bwd(
             gy.data_ptr(), gate.data_ptr(), h.data_ptr(), gh.data_ptr(), ggate.data_ptr(), ws.data_ptr(),
             gs, B, L, C, _dtype_code(gy), _dtype_code(gate), _dtype_code(h), _stream(h))
@@ -409,7 +427,7 @@ def gelu_tanh_fwd(x, tx=None):
     x, tx = _dense(x), _dense(tx)
     y = _empty(x.shape, x.dtype, x.device)
     ty = _empty(x.shape, x.dtype, x.device) if tx is not None else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_gelu_tanh_fwd(x.data_ptr(), _ptr(tx), y.data_ptr(), _ptr(ty), x.numel(), _dtype_code(x), _stream(x))
     _check(rc, "dmf_gelu_tanh_fwd")
     return y, ty
@@ -419,7 +437,7 @@ def gelu_tanh_bwd(gy, x):
     _same_dtype("gelu_tanh_bwd", x, gy)
     gy, x = _dense(gy), _dense(x)
     gx = _empty(x.shape, x.dtype, x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_gelu_tanh_bwd(gy.data_ptr(), x.data_ptr(), gx.data_ptr(), x.numel(), _dtype_code(x), _stream(x))
     _check(rc, "dmf_gelu_tanh_bwd")
     return gx
@@ -434,7 +452,7 @@ def rmsnorm_fwd(x, gain, tx=None, eps: float = 1e-6, jvp=False):
     B, L, H, D = x.shape
     y = _empty((B, L, H, D), x.dtype, x.device)
     ty = _empty((B, L, H, D), x.dtype, x.device) if jvp else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_rmsnorm_fwd(
             x.data_ptr(), _ptr(tx), gain.data_ptr(), y.data_ptr(), _ptr(ty), _strides(x, tx if tx is not None else x),
             B, L, H, D, float(eps), _dtype_code(x), _dtype_code(gain), _stream(x))
@@ -458,7 +476,7 @@ def rmsnorm_bwd(gy, x, gain, eps: float = 1e-6, out=None):
             raise ValueError("rmsnorm_bwd: `out` must have the shape of x")
     ggain = _empty((D,), gain.dtype, x.device)
     ws = _workspace(2, B, L, D, x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_rmsnorm_bwd(
             gy.data_ptr(), x.data_ptr(), gain.data_ptr(), gx.data_ptr(), ggain.data_ptr(), ws.data_ptr(), _strides(x, gx),
             B, L, H, D, float(eps), _dtype_code(x), _dtype_code(gain), _stream(x))
@@ -477,7 +495,7 @@ def colsum(x, out_dtype=None):
     out = _empty((C,), out_dtype or x.dtype, x.device)
     n = load().dmf_block_workspace_floats(3, 1, min(rows, 2 ** 31 - 1), C)
     ws = _empty((max(int(n), 1),), torch.float32, x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_colsum(x.data_ptr(), out.data_ptr(), ws.data_ptr(), rows, C, _dtype_code(x), _dtype_code(out), _stream(x))
     _check(rc, "dmf_colsum")
     return out
@@ -492,7 +510,7 @@ def silu_fwd(x, tx=None, out_dtype=None):
     out_dtype = out_dtype or x.dtype
     y = _empty(x.shape, out_dtype, x.device)
     ty = _empty(x.shape, out_dtype, x.device) if tx is not None else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_silu_fwd(x.data_ptr(), _ptr(tx), y.data_ptr(), _ptr(ty), x.numel(), _dtype_code(x), _dtype_code(y), _stream(x))
     _check(rc, "dmf_silu_fwd")
     return y, ty
@@ -501,7 +519,7 @@ def silu_fwd(x, tx=None, out_dtype=None):
 def silu_bwd(gy, x):
     gy, x = _dense(gy), _dense(x)
     gx = _empty(x.shape, x.dtype, x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_silu_bwd(gy.data_ptr(), x.data_ptr(), gx.data_ptr(), x.numel(), _dtype_code(x), _dtype_code(gy), _stream(x))
     _check(rc, "dmf_silu_bwd")
     return gx
@@ -524,7 +542,7 @@ def residual_ln_modulate_fwd(x, gate, h, shift, scale, tx=None, tgate=None, th=N
     z = _empty((B, L, C), out_dtype, x.device)
     ty = _empty((B, L, C), x.dtype, x.device) if jvp else None
     tz = _empty((B, L, C), out_dtype, x.device) if jvp else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = load().dmf_residual_ln_modulate_fwd(
             x.data_ptr(), _ptr(tx), mods[0][0].data_ptr(), _ptr(mods[1][0]), h.data_ptr(), _ptr(th),
             mods[2][0].data_ptr(), mods[3][0].data_ptr(), _ptr(mods[4][0]), _ptr(mods[5][0]),
