@@ -14,7 +14,11 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 import torch
 from torch._C import _functorch
 from torch._functorch.pyfunctorch import retrieve_all_functorch_interpreters as _interpreters
-from torch._functorch.pyfunctorch import temporarily_pop_interpreter_stack as _pop_interpreter
+try:   # private helpers of functorch: without them the operators go through functorch's own dispatch
+    from torch._functorch.pyfunctorch import temporarily_pop_interpreter_stack as _pop_interpreter
+    _HAVE_LEVEL_TOOLS = hasattr(_functorch, "_wrap_for_grad")
+except ImportError:
+    _pop_interpreter, _HAVE_LEVEL_TOOLS = None, False
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdmf_attn.so")
@@ -99,7 +103,7 @@ def _apply(fn_cls, args):
 
 
 # Call custom Functions below a single torch.func.jvp level instead of through it (module switch for A/B timing and tests).
-BASE_LEVEL_UNDER_JVP = True
+BASE_LEVEL_UNDER_JVP = _HAVE_LEVEL_TOOLS
 
 
 def run_function(fn_cls, *args):
