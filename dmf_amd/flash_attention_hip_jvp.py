@@ -89,6 +89,14 @@ def _is_dual_mode(*tensors) -> bool:
     return any(fwAD.unpack_dual(t).tangent is not None for t in tensors)
 
 
+def _padded_head_dim(d: int) -> int:
+    """The kernels' head dim that serves head dim ``d``: itself, or the next larger one."""
+    for n in _lib.SUPPORTED_HEAD_DIMS:
+        if n >= d:
+            return n
+    raise ValueError(f"head dim {d} exceeds the largest supported one ({_lib.SUPPORTED_HEAD_DIMS[-1]})")
+
+
 def flash_attn_func(q, k, v, softmax_scale=None):
     """Attention on (B, L, H, D) tensors; dual tensors in -> dual tensor out.
 
@@ -96,7 +104,17 @@ def flash_attn_func(q, k, v, softmax_scale=None):
     (models/flash_attention_2_jvp.py:294-319): under forward-mode AD the
     primals and tangents are unpacked (a missing tangent becomes zeros, :303-304),
     pushed through one fused kernel, and re-packed with ``fwAD.make_dual``.
+    Head dims without a kernel of their own (the reference covers them by splitting
+    and masking, models/triton_utils.py:22-45) are zero-padded to the next one that
+    has -- exact, since zero columns add nothing to the scores and give zero output
+    columns -- at the price of a padded copy of every operand.
     """
+    d = q.shape[-1]
+    dp = _padded_head_dim(d)
+    if dp != d:
+        scale = _default_scale(q, softmax_scale)
+        pad = lambda t: torch.nn.functional.pad(t, (0, dp - d))
+        return flash_attn_func(pad(q), pad(k), pad(v), scale)[..., :d]
     if _is_dual_mode(q, k, v):
         primals, tangents = [], []
         for t in (q, k, v):

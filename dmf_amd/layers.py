@@ -17,6 +17,7 @@ import torch.nn as nn
 from torch import Tensor
 
 from . import block_ops as fused
+from ._lib import SUPPORTED_HEAD_DIMS
 from .flash_attention_hip_jvp import flash_attn_func as hip_func
 from .flash_attention_hip_jvp import flash_attn_qknorm_qkvpacked_func as hip_qknorm_qkvpacked_func
 from .flash_attention_hip_jvp import flash_attn_qkvpacked_func as hip_qkvpacked_func
@@ -179,7 +180,8 @@ class Attention(nn.Module):
         self.proj = Linear(dim, dim, bias=proj_bias, block_ops=block_ops)
         self.attn = partial(attn_op, op=attn_func)
         # the 'hip' operator can take the projection output as it is (with or without qk-norm)
-        self.packed = _check_block_ops(block_ops) and attn_func == "hip"
+        # (head dims without a kernel of their own go through attn_op, which zero-pads them)
+        self.packed = _check_block_ops(block_ops) and attn_func == "hip" and self.head_dim in SUPPORTED_HEAD_DIMS
         self.qk_norm = qk_norm
 
     def forward(self, x: Tensor) -> Tensor:

@@ -229,8 +229,10 @@ def test_attention_module_hip_vs_base(qk_norm):
 
 def test_unsupported_head_dim_raises():
     q = torch.randn(1, 16, 2, 40, device=DEV)
-    with pytest.raises(RuntimeError, match="head dim"):
-        flash_attn_func(q, q, q)
+    with pytest.raises(RuntimeError, match="head dim"):      # the kernels themselves take the native head dims only
+        _lib.fwd(q, q, q, 40 ** -0.5)
+    with pytest.raises(ValueError, match="head dim"):        # and nothing pads beyond the largest one
+        flash_attn_func(q.repeat(1, 1, 1, 4), q.repeat(1, 1, 1, 4), q.repeat(1, 1, 1, 4))
     with pytest.raises(TypeError):
         flash_attn_func(q.half(), q.half(), q.half())
 
@@ -432,3 +434,37 @@ def test_huge_row_stride_takes_the_64bit_addressing_path():
     dq, dk, dv = _lib.bwd(cpu[6].to(DEV), q, k, v, o, lse, D ** -0.5)
     for got, ref in zip((dq, dk, dv), ao.base_attn_grads(*[t.float() for t in cpu[:3]], cpu[6].float())):
         assert ao.rel_l2(got.float().cpu(), ref) <= 2e-2
+
+
+@pytest.mark.parametrize("D", [16, 40, 48, 88, 104, 120])
+def test_other_head_dims_are_zero_padded(D):
+    """Head dims without a kernel of their own (the reference splits / masks them,
+    models/triton_utils.py:22-45): ``flash_attn_func`` pads them to the next native
+    size; outputs, tangents and gradients against the fp32 oracle, scale 1/sqrt(D) of
+    the real head dim."""
+    import dmf_amd
+    B, L, H = 2, 150, 3
+    q, k, v, tq, tk, tv, do = (t.to(DEV) for t in ao.make_inputs(B, L, H, D, seed=50 + D))
+    qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
+    o, to = torch.func.jvp(dmf_amd.flash_attn_func, (qg, kg, vg), (tq, tk, tv))
+    assert o.shape == (B, L, H, D)
+    o_ref, to_ref = ao.base_attn_jvp(*(t.cpu() for t in (q, k, v, tq, tk, tv)))
+    assert ao.rel_l2(o.cpu(), o_ref) <= TOL[torch.float32] and ao.rel_l2(to.cpu(), to_ref) <= TOL[torch.float32]
+    o.backward(do)
+    for got, ref in zip((qg.grad, kg.grad, vg.grad), ao.base_attn_grads(q.cpu(), k.cpu(), v.cpu(), do.cpu())):
+        assert ao.rel_l2(got.cpu(), ref) <= TOL[torch.float32]
+    with pytest.raises(ValueError):
+        dmf_amd.flash_attn_func(torch.zeros(1, 4, 1, 136, device=DEV), torch.zeros(1, 4, 1, 136, device=DEV), torch.zeros(1, 4, 1, 136, device=DEV))
+
+
+def test_attention_module_with_a_padded_head_dim():
+    """hidden 192 over 4 heads = head dim 48: the fused Attention module leaves the packed
+    fast path and still matches the naive operator."""
+    from dmf_amd.layers import Attention
+    torch.manual_seed(3)
+    a = Attention(192, num_heads=4, qkv_bias=True, qk_norm=True, attn_func="hip", block_ops="hip").to(DEV)
+    b = Attention(192, num_heads=4, qkv_bias=True, qk_norm=True, attn_func="base").to(DEV)
+    b.load_state_dict(a.state_dict())
+    assert not a.packed
+    x = torch.randn(2, 70, 192, device=DEV)
+    assert ao.rel_l2(a(x), b(x)) <= 1e-5
