@@ -74,9 +74,12 @@ def fake_kernels(monkeypatch):
     """Replace the three C-ABI calls by plain-torch stand-ins and count calls."""
     calls = {"fwd": 0, "fwd_jvp": 0, "bwd": 0}
 
+    def scaled(scale, d):   # the naive operator with the softmax scale the wrapper asks for instead of d ** -0.5
+        return lambda q, k, v: ao.base_attn(q * (scale * d ** 0.5), k, v)
+
     def fwd(q, k, v, scale, need_lse=True):
         calls["fwd"] += 1
-        return ao.base_attn(q, k, v).contiguous(), ao.lse_ref(q, k, scale).float()
+        return scaled(scale, q.shape[-1])(q, k, v).contiguous(), ao.lse_ref(q, k, scale).float()
 
     def fwd_jvp(q, k, v, tq, tk, tv, scale, need_dlse=False):
         calls["fwd_jvp"] += 1
@@ -88,7 +91,7 @@ def fake_kernels(monkeypatch):
     def bwd(dout, q, k, v, o, lse, scale):
         calls["bwd"] += 1
         with torch.enable_grad():   # autograd runs backward() with grad mode off
-            return ao.base_attn_grads(q, k, v, dout)
+            return ao.base_attn_grads(q, k, v, dout, fn=scaled(scale, q.shape[-1]))
 
     monkeypatch.setattr(_lib, "fwd", fwd)
     monkeypatch.setattr(_lib, "fwd_jvp", fwd_jvp)
@@ -165,7 +168,7 @@ def test_attention_module_feeds_packed_qkv_views(fake_kernels, monkeypatch):
     seen = []
     orig = _lib.fwd
     monkeypatch.setattr(_lib, "fwd", lambda q, k, v, s, need_lse=True: (seen.append((q.stride(), k.stride(), v.stride())), orig(q, k, v, s))[1])
-    B, L, H, D = 2, 6, 3, 8
+    B, L, H, D = 2, 6, 3, 32        # a head dim the kernels take as it is (others are padded into copies)
     x = torch.randn(B, L, H * D)
     for qk_norm in (False, True):
         m = Attention(H * D, num_heads=H, qkv_bias=True, qk_norm=qk_norm, attn_func="hip")
