@@ -12,8 +12,9 @@ bf16, q/k RMS-normalised), inputs resident in HBM.  Prints ONE JSON line:
                  timed on this box's host cores on a bounded slice of the
                  same workload
   extra          the other kernel-level figures (N=256 shape, backward,
-                 primal-only forward, the HBM-bound block-glue kernels) and
-                 DMFT forward+JVP / train-step images/s
+                 primal-only forward, the HBM-bound block-glue kernels), board
+                 power and shader clock while the attention kernels run, and
+                 end-to-end images/s of the DMFT / SiT steps and the sampler
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
 """
@@ -188,6 +189,75 @@ def device_probes():
     return out
 
 
+class _Telemetry:
+    """Samples the board's power draw and shader clock from sysfs (hwmon ``power1_input`` in microwatts, the
+    starred line of ``pp_dpm_sclk``) every few milliseconds on a thread while a block of GPU work runs."""
+
+    def __init__(self):
+        import glob
+        pw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
+        self.power_file = pw[0] if pw else None
+        dev = os.path.dirname(os.path.dirname(os.path.dirname(pw[0]))) if pw else None
+        self.sclk_file = os.path.join(dev, "pp_dpm_sclk") if dev and os.path.exists(os.path.join(dev, "pp_dpm_sclk")) else None
+        cap = pw[0].replace("power1_input", "power1_cap") if pw else None
+        self.cap_w = int(open(cap).read()) / 1e6 if cap and os.path.exists(cap) else None
+
+    def available(self):
+        return self.power_file is not None
+
+    def _sample(self):
+        p = int(open(self.power_file).read()) / 1e6
+        f = None
+        if self.sclk_file:
+            for line in open(self.sclk_file).read().splitlines():
+                if line.rstrip().endswith("*"):
+                    f = float(line.split(":")[1].strip().rstrip("*").strip().lower().replace("mhz", ""))
+        return p, f
+
+    def measure(self, fn, seconds=1.0):
+        """Run ``fn`` (which enqueues GPU work) repeatedly for about ``seconds`` and return mean / max power in watts
+        and the mean shader clock in MHz over the samples taken after the first quarter of the interval."""
+        import threading
+        import torch
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                try:
+                    samples.append((time.perf_counter(),) + self._sample())
+                except (OSError, ValueError, IndexError):
+                    pass
+                time.sleep(0.005)
+
+        th = threading.Thread(target=sampler, daemon=True)
+        t0 = time.perf_counter()
+        th.start()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+        stop.set()
+        th.join()
+        t1 = time.perf_counter()
+        keep = [x for x in samples if x[0] >= t0 + 0.25 * (t1 - t0)]
+        if not keep:
+            return None
+        clocks = [x[2] for x in keep if x[2] is not None]
+        return {"power_w_mean": sum(x[1] for x in keep) / len(keep), "power_w_max": max(x[1] for x in keep),
+                "sclk_mhz_mean": sum(clocks) / len(clocks) if clocks else None, "samples": len(keep)}
+
+
+def power_probes(fns):
+    """Board power and shader clock while each of the named GPU workloads runs for a second (None without sysfs access)."""
+    tel = _Telemetry()
+    if not tel.available():
+        return None
+    out = {"power_cap_w": tel.cap_w}
+    for label, fn in fns:
+        out[label] = tel.measure(fn)
+    return out
+
+
 def per_launch_stats(fn, iters=50):
     """Median and minimum duration (ms) of single launches, one HIP event pair per launch."""
     import torch
@@ -328,7 +398,14 @@ def main():
             progress(f"{wname}: fwd_jvp / fwd / bwd = " + " / ".join(f"{row[kd]['ms']:.4f}" for kd in ("fwd_jvp", "fwd", "bwd")) + " ms")
             del ins
         extra["device_probes"] = device_probes()
-        progress("device probes done")
+        zq = torch.zeros_like(q)
+        extra["power"] = power_probes([
+            ("attn_fwd_jvp_xl2_512px", lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)),
+            ("attn_fwd_jvp_xl2_512px_all_zero_inputs", lambda: _lib.fwd_jvp(zq, zq, zq, zq, zq, zq, scale)),
+            ("attn_bwd_xl2_512px", lambda: _lib.bwd(do, q, k, v, o, lse, scale)),
+        ])
+        del zq
+        progress("device probes done" + ("" if extra["power"] is None else f"; power {json.dumps(extra['power'])}"))
         extra["block_kernels"] = block_kernel_rows(dev)
         progress("block kernels done")
         try:
