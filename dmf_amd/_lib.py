@@ -118,7 +118,14 @@ def run_function(fn_cls, *args):
       unwrapped, ``apply`` runs below the level like the ordinary autograd node it is,
       and the outputs are wrapped for the level again (what functorch does for every
       built-in operator);
-    * otherwise (no transform, nested levels, ``vmap`` / ``grad``): plain ``apply``."""
+    * otherwise (no transform, nested levels, ``vmap`` / ``grad``): plain ``apply``.
+
+    Under ``torch.compile`` (the reference compiles the model it calls without JVP,
+    train_dmf.py:269-275) the call is a graph break: the kernels are reached through
+    ctypes, which a tracer cannot follow, so the operator runs eagerly between the
+    compiled pieces."""
+    if torch.compiler.is_compiling():
+        return _run_function_eagerly(fn_cls, *args)
     stack = _interpreters()
     if not stack:
         return _apply(fn_cls, args)
@@ -136,6 +143,11 @@ def run_function(fn_cls, *args):
         wrap = lambda o: _functorch._wrap_for_grad(o, level) if isinstance(o, torch.Tensor) else o
         return tuple(wrap(o) for o in outs) if isinstance(outs, tuple) else wrap(outs)
     return fn_cls.apply(*args)
+
+
+@torch.compiler.disable
+def _run_function_eagerly(fn_cls, *args):
+    return run_function(fn_cls, *args)
 
 
 _SIDE_STREAMS = {}

@@ -251,3 +251,30 @@ def test_frozen_low_precision_params_give_the_same_bits():
     with frozen_low_precision_params(m):
         harness.train_step(m, data)
     assert m.blocks[0].attn.qkv.weight.grad is not None and m.blocks[0].attn.qkv.weight.grad.dtype == torch.float32
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+@pytest.mark.parametrize("block_ops", ["torch", "hip"])
+def test_torch_compile_treats_the_operators_as_graph_breaks(backend, block_ops):
+    """The reference compiles the model it calls without JVP (train_dmf.py:269-275,
+    ``fullgraph=False``): under ``torch.compile`` the 'hip' operators run eagerly
+    between the compiled pieces -- same outputs and gradients as the eager model."""
+    dev = "cuda:0"
+    m = _small("hip", input_size=16, hidden_size=128, num_heads=2, qk_norm=True, block_ops=block_ops).to(dev)
+    z, t, r, y, _ = harness.synthetic_batch(4, dev, input_size=16)
+    ref = m(z, t, r, y)
+    ref.square().mean().backward()
+    g_ref = {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}
+    m.zero_grad(set_to_none=True)
+    torch._dynamo.reset()
+    cm = torch.compile(m, backend=backend, dynamic=True)
+    out = cm(z, t, r, y)
+    out.square().mean().backward()
+    assert ao.rel_l2(out, ref) <= 1e-5
+    for n, p in m.named_parameters():
+        if n in g_ref and float(g_ref[n].abs().max()) > 0:
+            assert ao.rel_l2(p.grad, g_ref[n]) <= 1e-4, n
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        assert ao.rel_l2(cm(z, t, r, y).float(), ref) <= 3e-2
+    torch._dynamo.reset()
