@@ -34,7 +34,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the fused fwd+JVP kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (each scaled by what the counter reads for a plain 1 GiB copy; summaries in profiles/attn_fwd_jvp_bf16_d72_*.txt)
-MEASURED_TRAFFIC_BYTES = {"xl2_512px": 1.2129e9, "xl2_256px": 1.2125e9}
+MEASURED_TRAFFIC_BYTES = {"xl2_512px": 1.2131e9, "xl2_256px": 1.2126e9}
 
 WORKLOADS = {
     # name: (B, H, N, D, qk_norm)
@@ -156,7 +156,7 @@ def roofline(name, ms):
     the machine balance (2.5 PFLOP/s / 8 TB/s = 312 FLOP/B), the HBM roof otherwise (N=256: 191 FLOP/B)."""
     B, H, N, D, _ = WORKLOADS[name]
     flops, nbytes = attn_flops(B, H, N, D, "fwd_jvp"), attn_bytes(B, H, N, D, "fwd_jvp")
-    common = {"traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8>"}
+    common = {"traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8, false>"}
     if flops / nbytes >= MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
         a = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": a / MFMA_BF16_PEAK_TFLOPS,
