@@ -94,16 +94,18 @@ def frozen_low_precision_params(model: nn.Module, dtype: torch.dtype = torch.bfl
     """While active, every fused ``Linear`` of ``model`` uses a copy of its parameters in
     ``dtype`` made once on entry, instead of the per-call casts of autocast -- for loops
     over frozen weights (sampling, evaluation, forward+JVP-only passes).  The caller must
-    not modify the parameters inside the context; results are those of autocast."""
+    not modify the parameters inside the context; results are those of autocast.  Contexts
+    nest: leaving an inner one puts back the copies of the outer one."""
     layers = [m for m in model.modules() if isinstance(m, Linear) and m.fused]
+    saved = [(m.lp_weight, m.lp_bias) for m in layers]
     try:
         for m in layers:
             m.lp_weight = m.weight.detach().to(dtype)
             m.lp_bias = None if m.bias is None else m.bias.detach().to(dtype)
         yield model
     finally:
-        for m in layers:
-            m.lp_weight = m.lp_bias = None
+        for m, (w, b) in zip(layers, saved):
+            m.lp_weight, m.lp_bias = w, b
 
 
 def modulate(x: Tensor, shift: Tensor, scale: Tensor) -> Tensor:

@@ -283,3 +283,16 @@ def test_run_function_below_a_single_jvp_level_matches_functorch_dispatch(monkey
     Scale.calls.clear()
     gx = torch.func.grad(lambda a: op(a, w.detach()).sum())(x)
     assert torch.allclose(gx, w.detach().expand_as(x)) and any(Scale.calls)
+
+
+def test_frozen_low_precision_params_nest_and_restore():
+    from dmf_amd.layers import Linear, frozen_low_precision_params
+    m = torch.nn.Sequential(Linear(8, 8, block_ops="hip"), Linear(8, 4, bias=False, block_ops="hip"), torch.nn.Linear(4, 4))
+    with frozen_low_precision_params(m):
+        outer = m[0].lp_weight
+        assert outer.dtype == torch.bfloat16 and torch.equal(outer, m[0].weight.detach().bfloat16())
+        assert m[1].lp_bias is None and m[1].lp_weight is not None and not hasattr(m[2], "lp_weight")
+        with frozen_low_precision_params(m, torch.float16):
+            assert m[0].lp_weight.dtype == torch.float16
+        assert m[0].lp_weight is outer              # the inner context put the outer copies back
+    assert m[0].lp_weight is None and m[0].lp_bias is None and m[1].lp_weight is None
