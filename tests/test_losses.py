@@ -354,3 +354,41 @@ def test_euler_sampler_bf16_model_fused_vs_base():
 
     out_g = euler_sampler(m, z, y, model_call=call, **args)
     assert sorted(graphs) == [8, 16] and ao.rel_l2(out_g, out) <= 1e-6
+
+
+@pytest.mark.gpu
+def test_graphed_dmf_step_follows_parameter_updates():
+    """A captured step must read the parameters as they are at replay time -- the
+    bf16 weight copies that the fused Linear layers share within a step are made
+    inside the graph -- so a few SGD updates give the same losses replayed as
+    eager, and the losses move."""
+    dev = "cuda:0"
+    kw = dict(input_size=16, hidden_size=128, depth=3, num_heads=2, dmf_depth=2)
+    m_e = _dmft("hip", block_ops="hip", **kw).to(dev)
+    m_g = _dmft("hip", block_ops="hip", **kw).to(dev)
+    m_g.load_state_dict(m_e.state_dict())
+    batch = harness.synthetic_loss_batch(8, dev, input_size=16)
+    guidance = dict(g_type="mg", omega=0.5)
+
+    def sgd(m, lr=0.5):
+        with torch.no_grad():
+            for p in m.parameters():
+                if p.grad is not None:
+                    p.add_(p.grad, alpha=-lr)
+
+    def step_g(*b):
+        m_g.zero_grad(set_to_none=True)
+        return harness.dmf_train_step(m_g, b, functorch=False, **guidance).detach()
+
+    graphed = harness.GraphedStep(step_g, *batch)
+    m_g.load_state_dict(m_e.state_dict())        # the warm-up calls did not update anything, but start from equal weights for sure
+    eager, replayed = [], []
+    for _ in range(4):
+        m_e.zero_grad(set_to_none=True)
+        eager.append(float(harness.dmf_train_step(m_e, batch, functorch=False, **guidance)))
+        sgd(m_e)
+        replayed.append(float(graphed(*batch)))
+        sgd(m_g)
+    assert abs(eager[-1] - eager[0]) > 1e-3 * abs(eager[0]), eager            # the updates matter
+    for a, b in zip(eager, replayed):
+        assert abs(a - b) <= 2e-3 * abs(a) + 1e-5, (eager, replayed)
