@@ -78,6 +78,32 @@ def unpatchify(x: Tensor, channels: int, patch: int) -> Tensor:
     return x.reshape(x.shape[0], channels, h * patch, w * patch)
 
 
+def reference_init_(model: nn.Module) -> nn.Module:
+    """The reference's initialisation of a DMFT or SiT (models/dmft.py:79-121, models/sit.py:84-120): Xavier-uniform
+    linears with zero biases (the patch projection counted as one), sin-cos positions, N(0, 0.02) label table and
+    timestep MLP, and zeros for every adaLN modulation, the output layer and the log-variance head -- which makes
+    every block an identity and the model output zero at step 0."""
+    for m in model.modules():
+        if isinstance(m, nn.Linear):
+            nn.init.xavier_uniform_(m.weight)
+            if m.bias is not None:
+                nn.init.zeros_(m.bias)
+    grid = int(model.num_patches ** 0.5)
+    model.pos_embed.data.copy_(torch.from_numpy(get_2d_sincos_pos_embed(model.pos_embed.shape[-1], grid)).float().unsqueeze(0))
+    proj = model.x_embedder.proj
+    nn.init.xavier_uniform_(proj.weight.data.view(proj.weight.shape[0], -1))
+    nn.init.zeros_(proj.bias)
+    for table in (model.y_embedder.embedding_table.weight, model.t_embedder.mlp[0].weight, model.t_embedder.mlp[2].weight):
+        nn.init.normal_(table, std=0.02)
+    zeroed = [blk.adaLN_modulation[-1] for blk in model.blocks] + [model.final_layer.adaLN_modulation[-1], model.final_layer.linear]
+    if getattr(model, "use_logvar", False):
+        zeroed.append(model.logvar_linear)
+    for layer in zeroed:
+        nn.init.zeros_(layer.weight)
+        nn.init.zeros_(layer.bias)
+    return model
+
+
 def trunc_normal_init_(model: nn.Module, std: float = 0.02, seed: int = 0) -> nn.Module:
     """Benchmark initialisation: every weight matrix / embedding ~ truncated
     N(0, std) (cut at 2 std), biases zero.  With the reference's zero-gate
@@ -130,33 +156,7 @@ class DMFT(nn.Module):
         self.initialize_weights()
 
     def initialize_weights(self) -> None:
-        """The reference's initialisation (models/dmft.py:79-121): Xavier linears,
-        N(0, 0.02) embeddings, and zeroed adaLN gates / output layer -- which makes
-        every block an identity and the output zero at step 0."""
-        def _basic_init(m):
-            if isinstance(m, nn.Linear):
-                nn.init.xavier_uniform_(m.weight)
-                if m.bias is not None:
-                    nn.init.constant_(m.bias, 0)
-        self.apply(_basic_init)
-        pe = get_2d_sincos_pos_embed(self.pos_embed.shape[-1], int(self.num_patches ** 0.5))
-        self.pos_embed.data.copy_(torch.from_numpy(pe).float().unsqueeze(0))
-        w = self.x_embedder.proj.weight.data
-        nn.init.xavier_uniform_(w.view([w.shape[0], -1]))
-        nn.init.constant_(self.x_embedder.proj.bias, 0)
-        nn.init.normal_(self.y_embedder.embedding_table.weight, std=0.02)
-        nn.init.normal_(self.t_embedder.mlp[0].weight, std=0.02)
-        nn.init.normal_(self.t_embedder.mlp[2].weight, std=0.02)
-        for block in self.blocks:
-            nn.init.constant_(block.adaLN_modulation[-1].weight, 0)
-            nn.init.constant_(block.adaLN_modulation[-1].bias, 0)
-        nn.init.constant_(self.final_layer.adaLN_modulation[-1].weight, 0)
-        nn.init.constant_(self.final_layer.adaLN_modulation[-1].bias, 0)
-        nn.init.constant_(self.final_layer.linear.weight, 0)
-        nn.init.constant_(self.final_layer.linear.bias, 0)
-        if self.use_logvar:
-            nn.init.constant_(self.logvar_linear.weight, 0)
-            nn.init.constant_(self.logvar_linear.bias, 0)
+        reference_init_(self)
 
     def init_trunc_normal_(self, std: float = 0.02, seed: int = 0) -> "DMFT":
         return trunc_normal_init_(self, std, seed)

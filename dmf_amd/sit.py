@@ -16,9 +16,8 @@ from functools import partial
 import torch
 import torch.nn as nn
 
-from .dmft import PatchEmbed, chained_blocks, trunc_normal_init_, unpatchify
-from .layers import (DiTBlock, FinalLayer, LabelEmbedder, Linear, SiLU, TimestepEmbedder, _check_block_ops,
-                     get_2d_sincos_pos_embed)
+from .dmft import PatchEmbed, chained_blocks, reference_init_, trunc_normal_init_, unpatchify
+from .layers import DiTBlock, FinalLayer, LabelEmbedder, Linear, SiLU, TimestepEmbedder, _check_block_ops
 
 
 def build_mlp(hidden_size: int, projector_dim: int, z_dim: int, block_ops: str = "torch") -> nn.Sequential:
@@ -54,29 +53,7 @@ class SiT(nn.Module):
         self.initialize_weights()
 
     def initialize_weights(self) -> None:
-        """The reference's initialisation (models/sit.py:84-120): Xavier linears,
-        N(0, 0.02) embeddings, zeroed adaLN gates and output layer."""
-        def _basic_init(m):
-            if isinstance(m, nn.Linear):
-                nn.init.xavier_uniform_(m.weight)
-                if m.bias is not None:
-                    nn.init.constant_(m.bias, 0)
-        self.apply(_basic_init)
-        pe = get_2d_sincos_pos_embed(self.pos_embed.shape[-1], int(self.num_patches ** 0.5))
-        self.pos_embed.data.copy_(torch.from_numpy(pe).float().unsqueeze(0))
-        w = self.x_embedder.proj.weight.data
-        nn.init.xavier_uniform_(w.view([w.shape[0], -1]))
-        nn.init.constant_(self.x_embedder.proj.bias, 0)
-        nn.init.normal_(self.y_embedder.embedding_table.weight, std=0.02)
-        nn.init.normal_(self.t_embedder.mlp[0].weight, std=0.02)
-        nn.init.normal_(self.t_embedder.mlp[2].weight, std=0.02)
-        for block in self.blocks:
-            nn.init.constant_(block.adaLN_modulation[-1].weight, 0)
-            nn.init.constant_(block.adaLN_modulation[-1].bias, 0)
-        nn.init.constant_(self.final_layer.adaLN_modulation[-1].weight, 0)
-        nn.init.constant_(self.final_layer.adaLN_modulation[-1].bias, 0)
-        nn.init.constant_(self.final_layer.linear.weight, 0)
-        nn.init.constant_(self.final_layer.linear.bias, 0)
+        reference_init_(self)
 
     def init_trunc_normal_(self, std: float = 0.02, seed: int = 0) -> "SiT":
         return trunc_normal_init_(self, std, seed)
