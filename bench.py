@@ -216,7 +216,7 @@ class _Telemetry:
                     f = float(line.split(":")[1].strip().rstrip("*").strip().lower().replace("mhz", ""))
         return p, f
 
-    def measure(self, fn, seconds=1.0):
+    def measure(self, fn, seconds=1.0, burst=20):
         """Run ``fn`` (which enqueues GPU work) repeatedly for about ``seconds`` and return mean / max power in watts
         and the mean shader clock in MHz over the samples taken after the first quarter of the interval."""
         import threading
@@ -235,7 +235,7 @@ class _Telemetry:
         t0 = time.perf_counter()
         th.start()
         while time.perf_counter() - t0 < seconds:
-            for _ in range(20):
+            for _ in range(burst):
                 fn()
             torch.cuda.synchronize()
         stop.set()
@@ -257,6 +257,17 @@ def power_probes(fns):
     out = {"power_cap_w": tel.cap_w}
     for label, fn in fns:
         out[label] = tel.measure(fn)
+    probe = os.path.join(ROOT, "dmf_amd", "libdmf_probe.so")
+    if os.path.exists(probe):   # the register-only MFMA loop of device_probes(): what pure matrix work draws (each call is synchronous)
+        import ctypes
+        lib = ctypes.CDLL(probe)
+        lib.dmf_probe_mfma_tflops.restype = ctypes.c_float
+        lib.dmf_probe_mfma_tflops.argtypes = [ctypes.c_int, ctypes.c_int]
+        for label, rnd in (("mfma_loop_random_operands", 1), ("mfma_loop_constant_operands", 0)):
+            rates = []
+            out[label] = tel.measure(lambda: rates.append(lib.dmf_probe_mfma_tflops(rnd, 20000)), burst=1)
+            if out[label] is not None and rates:
+                out[label]["tflops_mean"] = sum(rates) / len(rates)
     return out
 
 
