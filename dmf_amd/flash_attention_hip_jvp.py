@@ -89,6 +89,48 @@ def _is_dual_mode(*tensors) -> bool:
     return any(fwAD.unpack_dual(t).tangent is not None for t in tensors)
 
 
+# ---- the primal operator as a registered custom op: what torch.compile traces instead of the ctypes calls ------------
+# (forward + backward on the primal output, no tangents: the reference compiles only the model it calls without JVP,
+#  train_dmf.py:269-275; in eager mode nothing goes through here)
+
+@torch.library.custom_op("dmf_amd::attn_fwd", mutates_args=())
+def _attn_fwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> tuple[torch.Tensor, torch.Tensor]:
+    return _lib.fwd(q, k, v, scale, need_lse=True)
+
+
+@_attn_fwd_op.register_fake
+def _(q, k, v, scale):
+    B, Lq, H, D = q.shape
+    return q.new_empty((B, Lq, H, D)), q.new_empty((B, H, Lq), dtype=torch.float32)
+
+
+@torch.library.custom_op("dmf_amd::attn_bwd", mutates_args=())
+def _attn_bwd_op(dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
+                 scale: float) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _lib.bwd(dout, q, k, v, o, lse, scale)
+
+
+@_attn_bwd_op.register_fake
+def _(dout, q, k, v, o, lse, scale):
+    return tuple(t.new_empty(t.shape) for t in (q, k, v))
+
+
+def _attn_op_setup(ctx, inputs, output):
+    q, k, v, scale = inputs
+    o, lse = output
+    ctx.save_for_backward(q, k, v, o, lse)
+    ctx.scale = scale
+
+
+def _attn_op_backward(ctx, dout, dlse_unused):
+    q, k, v, o, lse = ctx.saved_tensors
+    dq, dk, dv = torch.ops.dmf_amd.attn_bwd(dout, q, k, v, o, lse, ctx.scale)
+    return dq, dk, dv, None
+
+
+_attn_fwd_op.register_autograd(_attn_op_backward, setup_context=_attn_op_setup)
+
+
 def _padded_head_dim(d: int) -> int:
     """The kernels' head dim that serves head dim ``d``: itself, or the next larger one."""
     for n in _lib.SUPPORTED_HEAD_DIMS:
@@ -115,6 +157,9 @@ def flash_attn_func(q, k, v, softmax_scale=None):
         scale = _default_scale(q, softmax_scale)
         pad = lambda t: torch.nn.functional.pad(t, (0, dp - d))
         return flash_attn_func(pad(q), pad(k), pad(v), scale)[..., :d]
+    if torch.compiler.is_compiling():
+        # traced by torch.compile: one opaque operator in the graph (no forward-AD inside compiled code)
+        return torch.ops.dmf_amd.attn_fwd(q, k, v, float(_default_scale(q, softmax_scale)))[0]
     if _is_dual_mode(q, k, v):
         primals, tangents = [], []
         for t in (q, k, v):

@@ -468,3 +468,18 @@ def test_attention_module_with_a_padded_head_dim():
     assert not a.packed
     x = torch.randn(2, 70, 192, device=DEV)
     assert ao.rel_l2(a(x), b(x)) <= 1e-5
+
+
+def test_registered_operators_pass_opcheck():
+    """``dmf_amd::attn_fwd`` / ``attn_bwd`` (what torch.compile traces): schema, fake
+    tensor implementation, autograd registration and AOT dispatch, on packed-qkv views."""
+    import dmf_amd  # noqa: F401  (registers the operators)
+    qkv = torch.randn(2, 40, 3, 3, 64, device=DEV, requires_grad=True)
+    q, k, v = qkv.unbind(2)
+    res = torch.library.opcheck(torch.ops.dmf_amd.attn_fwd.default, (q, k, v, 0.125))
+    assert set(res.values()) == {"SUCCESS"}, res
+    o, lse = torch.ops.dmf_amd.attn_fwd(q.detach(), k.detach(), v.detach(), 0.125)
+    res = torch.library.opcheck(torch.ops.dmf_amd.attn_bwd.default, (torch.randn_like(o), q.detach(), k.detach(), v.detach(), o, lse, 0.125))
+    assert set(res.values()) == {"SUCCESS"}, res
+    o2, lse2 = _lib.fwd(q.detach(), k.detach(), v.detach(), 0.125)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
