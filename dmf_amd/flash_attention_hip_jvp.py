@@ -19,6 +19,8 @@ a second pass of the fused kernel over the saved primals.
 """
 from __future__ import annotations
 
+import warnings
+
 import torch
 import torch.autograd.forward_ad as fwAD
 
@@ -131,6 +133,9 @@ def _attn_op_backward(ctx, dout, dlse_unused):
 _attn_fwd_op.register_autograd(_attn_op_backward, setup_context=_attn_op_setup)
 
 
+_warned_fp16 = False
+
+
 def _padded_head_dim(d: int) -> int:
     """The kernels' head dim that serves head dim ``d``: itself, or the next larger one."""
     for n in _lib.SUPPORTED_HEAD_DIMS:
@@ -149,8 +154,18 @@ def flash_attn_func(q, k, v, softmax_scale=None):
     Head dims without a kernel of their own (the reference covers them by splitting
     and masking, models/triton_utils.py:22-45) are zero-padded to the next one that
     has -- exact, since zero columns add nothing to the scores and give zero output
-    columns -- at the price of a padded copy of every operand.
+    columns -- at the price of a padded copy of every operand.  fp16 operands (the
+    reference's ``--mixed-precision fp16`` / ``--dtype fp16``) have no kernels of their
+    own either: they are computed by the fp32 kernels and rounded back to fp16, which
+    is exact to fp16 rounding but an order of magnitude slower than bf16 (warned once).
     """
+    if q.dtype == torch.float16:
+        global _warned_fp16
+        if not _warned_fp16:
+            _warned_fp16 = True
+            warnings.warn("dmf_amd attention: fp16 operands are computed by the fp32 kernels (correct, but about ten times "
+                          "slower than bf16 on this device); use bf16 for speed", stacklevel=2)
+        return flash_attn_func(q.float(), k.float(), v.float(), _default_scale(q, softmax_scale)).to(torch.float16)
     d = q.shape[-1]
     dp = _padded_head_dim(d)
     if dp != d:

@@ -233,8 +233,28 @@ def test_unsupported_head_dim_raises():
         _lib.fwd(q, q, q, 40 ** -0.5)
     with pytest.raises(ValueError, match="head dim"):        # and nothing pads beyond the largest one
         flash_attn_func(q.repeat(1, 1, 1, 4), q.repeat(1, 1, 1, 4), q.repeat(1, 1, 1, 4))
+    with pytest.raises(TypeError):                           # the kernels take fp32 and bf16 only ...
+        _lib.fwd(q.half(), q.half(), q.half(), 40 ** -0.5)
     with pytest.raises(TypeError):
-        flash_attn_func(q.half(), q.half(), q.half())
+        flash_attn_func(q.double(), q.double(), q.double())
+
+
+def test_fp16_operands_go_through_the_fp32_kernels():
+    """... and fp16 operands (``--mixed-precision fp16``) are upcast to the fp32 kernels by
+    the wrapper and rounded back: fp16 in, fp16 out, tangents and gradients included."""
+    import warnings
+    q, k, v, tq, tk, tv, do = (t.to(DEV).half() for t in ao.make_inputs(2, 70, 3, 64, seed=77))
+    qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        o, to = torch.func.jvp(flash_attn_func, (qg, kg, vg), (tq, tk, tv))
+    assert o.dtype == torch.float16 and to.dtype == torch.float16
+    f = lambda t: t.float().cpu()
+    o_ref, to_ref = ao.base_attn_jvp(f(q), f(k), f(v), f(tq), f(tk), f(tv))
+    assert ao.rel_l2(f(o), o_ref) <= 1e-3 and ao.rel_l2(f(to), to_ref) <= 1e-3          # fp16 rounding of the results
+    o.backward(do)
+    for got, ref in zip((qg.grad, kg.grad, vg.grad), ao.base_attn_grads(f(q), f(k), f(v), f(do))):
+        assert got.dtype == torch.float16 and ao.rel_l2(f(got), ref) <= 2e-3
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
