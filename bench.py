@@ -169,11 +169,11 @@ def roofline(name, ms):
 
 
 def device_probes():
-    """Practical ceilings of this device (dmf_amd/csrc/probes.hip): sustained bf16 MFMA rate from a register-only
+    """Practical ceilings of this device (bench_probes.hip): sustained bf16 MFMA rate from a register-only
     loop with constant and with random operand bits (power-limited clocks), and the bandwidth of a math-free kernel
     with the operator's row access pattern at the N=256 workload."""
     import ctypes
-    path = os.path.join(ROOT, "dmf_amd", "libdmf_probe.so")
+    path = os.path.join(ROOT, "libbench_probes.so")
     if not os.path.exists(path):
         return None
     lib = ctypes.CDLL(path)
@@ -257,7 +257,7 @@ def power_probes(fns):
     out = {"power_cap_w": tel.cap_w}
     for label, fn in fns:
         out[label] = tel.measure(fn)
-    probe = os.path.join(ROOT, "dmf_amd", "libdmf_probe.so")
+    probe = os.path.join(ROOT, "libbench_probes.so")
     if os.path.exists(probe):   # the register-only MFMA loop of device_probes(): what pure matrix work draws (each call is synchronous)
         import ctypes
         lib = ctypes.CDLL(probe)

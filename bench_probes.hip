@@ -1,4 +1,4 @@
-// Measurement aids for bench.py (not part of the attention ABI).
+// Measurement aids for bench.py (not part of the attention library or its ABI; built into libbench_probes.so).
 //
 // dmf_probe_mfma_tflops: sustained rate of v_mfma_f32_32x32x16_bf16 on this
 // device from a register-only loop, with constant or with random operand bits.

@@ -9,6 +9,7 @@ from __future__ import annotations
 import contextlib
 import ctypes
 import os
+import warnings
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 
 import torch
@@ -145,6 +146,15 @@ def run_function(fn_cls, *args):
     return fn_cls.apply(*args)
 
 
+def plain_inference(*tensors) -> bool:
+    """True when a primal-only call needs nothing kept for later: no gradient can be asked for (grad mode off, or no
+    operand requires one) and no functorch transform is active.  Such calls (sampling, guidance targets) run the
+    kernels directly -- no autograd node, no log-sum-exp output."""
+    if torch.compiler.is_compiling() or _interpreters():
+        return False
+    return not (torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors))
+
+
 @torch.compiler.disable
 def _run_function_eagerly(fn_cls, *args):
     return run_function(fn_cls, *args)
@@ -182,7 +192,22 @@ def _prep(t: torch.Tensor) -> torch.Tensor:
     t = _raw(t)
     eb = t.element_size()
     ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all((s * eb) % 16 == 0 for s in t.stride()[:-1])
-    return t if ok else _raw(t.contiguous())
+    if ok:
+        return t
+    # A layout the kernels cannot read in place costs a full extra HBM round trip per operand: count it and say so once.
+    global relayout_copies
+    relayout_copies += 1
+    if relayout_copies == 1:
+        warnings.warn(
+            f"dmf_amd: operand with shape {tuple(t.shape)}, strides {tuple(t.stride())} and data pointer "
+            f"{'aligned' if t.data_ptr() % 16 == 0 else 'not aligned'} to 16 bytes is copied to a contiguous buffer before "
+            "the kernel runs (needs unit last-dim stride and 16-byte aligned rows); further copies are counted in "
+            "dmf_amd._lib.relayout_copies without a warning", RuntimeWarning, stacklevel=3)
+    return _raw(t.contiguous())
+
+
+# Number of operands _prep had to copy because of their layout since import (0 on the model path: packed-qkv views are read in place).
+relayout_copies = 0
 
 
 def _strides(*tensors) -> ctypes.Array:

@@ -13,7 +13,6 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdmf_attn.so")
-PROBE_LIB = os.path.join(HERE, "libdmf_probe.so")
 SOURCES = ["attn_fwd.hip", "attn_fwd_bf16.hip", "attn_bwd.hip", "attn_bwd_bf16.hip", "dmf_attn_abi.hip", "block_ops.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -47,13 +46,6 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
-    # measurement aids used by bench.py only (sustained MFMA rate, row-streaming bandwidth); separate library, not part of the ABI
-    probe_obj = _compile("probes.hip", objdir)
-    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB, probe_obj], capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"link failed:\n{r.stderr}")
-    if verbose:
-        print(f"built {PROBE_LIB}")
     return LIB
 
 

@@ -254,10 +254,8 @@ static int launch_bwd_t(const BwdParams& p, int BH, hipStream_t stream) {
   static bool lds_ok1[64] = {}, lds_ok2[64] = {};
   if (!ensure_dynamic_lds(k1, smem, lds_ok1) || !ensure_dynamic_lds(k2, smem, lds_ok2)) return -7;
   const uint32_t nqb = (p.Lq + 127) / 128, nkb = (p.Lkv + 127) / 128;
-  hipLaunchKernelGGL(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
-  if (hipGetLastError() != hipSuccess) return -7;
-  hipLaunchKernelGGL(k2, dim3(nkb * (uint32_t)BH), dim3(256), smem, stream, p);
-  return hipGetLastError() == hipSuccess ? 0 : -7;
+  if (int rc = launch_kernel(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p)) return rc;
+  return launch_kernel(k2, dim3(nkb * (uint32_t)BH), dim3(256), smem, stream, p);
 }
 
 template <typename T>

@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   const uint32_t rb_q = (uint32_t)p.st[1][1] * 2, rb_do = (uint32_t)p.st[0][1] * 2;
   const __amdgpu_buffer_rsrc_t rs_q = make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(1), rb_q, p.Lq, D * 2);
   const __amdgpu_buffer_rsrc_t rs_do = make_rows_rsrc(reinterpret_cast<const T*>(p.dout) + base(0), rb_do, p.Lq, D * 2);
-  // per-row statistics: padded query rows read lse = delta = 0; their Q and dout rows are zero, so they add nothing
+  // per-row statistics: padded query rows read lse = delta = 0 and are masked where P is formed
   const __amdgpu_buffer_rsrc_t rs_lse = make_rows_rsrc(p.lse + (int64_t)bh * p.Lq, 4, p.Lq, 4);
   const __amdgpu_buffer_rsrc_t rs_dl = make_rows_rsrc(p.delta + (int64_t)bh * p.Lq, 4, p.Lq, 4);
   auto issue = [&](int it) {
@@ -284,8 +284,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
         mma_chunk<T>(dP, oc[c & 1], Vr[c]);
       });
     }
-    // ---- P = exp2(S - lse*log2e), dS = P * (dP - delta)
+    // ---- P = exp2(S - lse*log2e), dS = P * (dP - delta).  Query rows past Lq are switched off here (P = 0): the
+    //      bounds check zero-fills them only when consecutive rows are distinct addresses, and a broadcast operand
+    //      (row stride 0, e.g. the gradient of a sum over the sequence) aliases them onto row 0 instead.
     f32x16 Pm, dS;
+    const bool qtail = (it + 1) * 32 > p.Lq;   // wave-uniform
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const f32x4 l4 = *reinterpret_cast<const f32x4*>(stat + j * 8 + 4 * g);
@@ -293,8 +296,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int i = 4 * j + e;
-        Pm[i] = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
-        dS[i] = Pm[i] * (dP[i] - d4[e]);
+        float pr = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
+        if (qtail && it * 32 + acc_row(i, g) >= p.Lq) pr = 0.f;
+        Pm[i] = pr;
+        dS[i] = pr * (dP[i] - d4[e]);
       }
     }
     // ---- dV^T += dout^T P ; dK^T += Q^T dS
@@ -361,10 +366,8 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
   static bool lds_ok1[64] = {}, lds_ok2[64] = {};
   if (!ensure_dynamic_lds(k1, smem1, lds_ok1) || !ensure_dynamic_lds(k2, smem, lds_ok2)) return -7;
   const uint32_t nqb = (p.Lq + 127) / 128, nkb = (p.Lkv + 127) / 128;
-  hipLaunchKernelGGL(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem1, stream, p);
-  if (hipGetLastError() != hipSuccess) return -7;
-  hipLaunchKernelGGL(k2, dim3(nkb * (uint32_t)BH), dim3(256), smem, stream, p);
-  return hipGetLastError() == hipSuccess ? 0 : -7;
+  if (int rc = launch_kernel(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem1, stream, p)) return rc;
+  return launch_kernel(k2, dim3(nkb * (uint32_t)BH), dim3(256), smem, stream, p);
 }
 
 // Returns 1 if there is no tuned kernel for the case (caller uses the generic ones).

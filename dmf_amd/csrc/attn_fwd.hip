@@ -202,8 +202,7 @@ static int launch_fwd_t(const FwdParams& p, int BH, hipStream_t stream) {
   static bool lds_ok[64] = {};
   if (!ensure_dynamic_lds(kern, smem, lds_ok)) return -7;
   const uint32_t nqb = (p.Lq + 127) / 128;
-  hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
-  return hipGetLastError() == hipSuccess ? 0 : -7;
+  return launch_kernel(kern, dim3(nqb * (uint32_t)BH), dim3(256), smem, stream, p);
 }
 
 template <typename T, bool JVP>

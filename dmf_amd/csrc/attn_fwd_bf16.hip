@@ -18,7 +18,6 @@
 #include "attn_common.h"
 #include "attn_kernels.h"
 #include <algorithm>
-#include <cstdlib>
 
 namespace dmf {
 
@@ -406,8 +405,7 @@ static int launch_fast_q(const FwdParams& p, int BH, hipStream_t stream) {
   static bool lds_ok[64] = {};
   if (!ensure_dynamic_lds(kern, smem, lds_ok)) return -7;
   const uint32_t nqb = (p.Lq + 32 * NW - 1) / (32 * NW);
-  hipLaunchKernelGGL(kern, dim3(nqb * (uint32_t)BH), dim3(64 * NW), smem, stream, p);
-  return hipGetLastError() == hipSuccess ? 0 : -7;
+  return launch_kernel(kern, dim3(nqb * (uint32_t)BH), dim3(64 * NW), smem, stream, p);
 }
 
 template <int D, bool JVP, int NW>
@@ -419,13 +417,8 @@ static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
   return launch_fast_q<D, JVP, NW, false>(p, BH, stream);
 }
 
-// Work-group width policy (256-row work-groups when the sequence fills them).
-static bool fwd_wide_workgroups(int Lq) {
-  static const int force = [] { const char* e = getenv("DMF_ATTN_FWD_NW"); return e ? atoi(e) : 0; }();
-  if (force == 4) return false;
-  if (force == 8) return true;
-  return Lq > 128;
-}
+// Work-group width policy: 256-row work-groups (one per CU, half the tile traffic per FLOP) when the sequence fills them.
+static bool fwd_wide_workgroups(int Lq) { return Lq > 128; }
 
 // Returns 1 if this translation unit has no kernel for the case (caller falls
 // back to the generic kernel), else 0 / negative error code.

@@ -48,6 +48,16 @@ inline bool ensure_dynamic_lds(K kernel, int bytes, bool (&done)[64]) {
   return true;
 }
 
+
+// Launch `kernel(params)` and return 0 or -7 (DMF_ATTN_ELAUNCH).  The status is the one hipLaunchKernel returns for
+// this launch; the process-wide "last error" is neither read nor cleared, so an error left behind by somebody
+// else's earlier call is not reported as a failure of this library (nor hidden from its owner).
+template <typename P>
+inline int launch_kernel(void (*kernel)(P), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, P params) {
+  void* args[] = {&params};
+  return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, args, lds_bytes, stream) == hipSuccess ? 0 : -7;
+}
+
 // Return 0 or a negative DMF_ATTN_E* code.
 int launch_fwd(const FwdParams& p, int BH, int D, bool bf16, bool jvp, hipStream_t stream);
 // Building blocks of launch_fwd: the generic kernels (fp32 and bf16, any length)

@@ -16,6 +16,7 @@
 
 #include "../../include/dmf_block.h"
 #include "attn_common.h"
+#include "attn_kernels.h"
 
 namespace dmf {
 namespace blk {
@@ -708,7 +709,6 @@ inline int ebytes(int d) { return d == DMF_ATTN_BF16 ? 2 : 4; }
 inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 inline int nchunks(int L) { return (L + kChunkRows - 1) / kChunkRows; }
 
-inline int launch_status() { return hipGetLastError() == hipSuccess ? DMF_ATTN_OK : DMF_ATTN_ELAUNCH; }
 
 // Shape checks shared by the (B, L, C) entry points.
 inline int check_blc(int B, int L, int C) {
@@ -728,12 +728,11 @@ inline int check_mod(const void* p, int64_t stride, int dtype, bool required) {
 template <typename F>
 inline int dispatch_nv(int C, F&& f) {
   switch ((C + 511) / 512) {
-    case 1: f(std::integral_constant<int, 1>{}); break;
-    case 2: f(std::integral_constant<int, 2>{}); break;
-    case 3: f(std::integral_constant<int, 3>{}); break;
-    default: f(std::integral_constant<int, 4>{}); break;
+    case 1: return f(std::integral_constant<int, 1>{});
+    case 2: return f(std::integral_constant<int, 2>{});
+    case 3: return f(std::integral_constant<int, 3>{});
+    default: return f(std::integral_constant<int, 4>{});
   }
-  return launch_status();
 }
 
 inline int reduce_partials(const float* partial, void* out0, void* out1, int B, int nchunk, int K, int C, int obf,
@@ -748,8 +747,7 @@ inline int reduce_partials(const float* partial, void* out0, void* out1, int B, 
   r.C = C;
   r.obf = obf;
   const unsigned grid = static_cast<unsigned>((r.total + 63) / 64);
-  hipLaunchKernelGGL(reduce_partials_kernel, dim3(grid), dim3(kThreads), 0, s, r);
-  return launch_status();
+  return launch_kernel(reduce_partials_kernel, dim3(grid), dim3(kThreads), 0, s, r);
 }
 
 template <int ACT>
@@ -764,16 +762,16 @@ inline int act_impl(const void* x, const void* t, void* y, void* ty, int64_t n, 
   p.xbf = x_dtype == DMF_ATTN_BF16; p.ybf = y_dtype == DMF_ATTN_BF16;
   const unsigned grid = static_cast<unsigned>((p.total + kThreads - 1) / kThreads);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (mode == 0) hipLaunchKernelGGL((act_kernel<ACT, 0>), dim3(grid), dim3(kThreads), 0, s, p);
-  else if (mode == 1) hipLaunchKernelGGL((act_kernel<ACT, 1>), dim3(grid), dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL((act_kernel<ACT, 2>), dim3(grid), dim3(kThreads), 0, s, p);
-  return launch_status();
+  if (mode == 0) return launch_kernel(act_kernel<ACT, 0>, dim3(grid), dim3(kThreads), 0, s, p);
+  if (mode == 1) return launch_kernel(act_kernel<ACT, 1>, dim3(grid), dim3(kThreads), 0, s, p);
+  return launch_kernel(act_kernel<ACT, 2>, dim3(grid), dim3(kThreads), 0, s, p);
 }
 
 }  // namespace blk
 }  // namespace dmf
 
 using namespace dmf::blk;
+using dmf::launch_kernel;
 
 extern "C" {
 
@@ -809,8 +807,8 @@ int dmf_ln_modulate_fwd(const void* x, const void* tx, const void* shift, const 
   hipStream_t s = static_cast<hipStream_t>(stream);
   return dispatch_nv(C, [&](auto nv) {
     constexpr int NV = decltype(nv)::value;
-    if (ty) hipLaunchKernelGGL((ln_modulate_fwd_kernel<NV, true>), dim3(grid), dim3(kThreads), 0, s, p);
-    else hipLaunchKernelGGL((ln_modulate_fwd_kernel<NV, false>), dim3(grid), dim3(kThreads), 0, s, p);
+    if (ty) return launch_kernel(ln_modulate_fwd_kernel<NV, true>, dim3(grid), dim3(kThreads), 0, s, p);
+    return launch_kernel(ln_modulate_fwd_kernel<NV, false>, dim3(grid), dim3(kThreads), 0, s, p);
   });
 }
 
@@ -833,7 +831,7 @@ int dmf_ln_modulate_bwd(const void* gy, const void* x, const void* scale, const 
   const int rc = dispatch_nv(C, [&](auto nv) {
     constexpr int NV = decltype(nv)::value;
     constexpr size_t lds = (kWaves - 1) * 2 * NV * 512 * sizeof(float);
-    hipLaunchKernelGGL((ln_modulate_bwd_kernel<NV>), dim3(grid), dim3(kThreads), lds, s, p);
+    return launch_kernel(ln_modulate_bwd_kernel<NV>, dim3(grid), dim3(kThreads), lds, s, p);
   });
   if (rc) return rc;
   return reduce_partials(workspace, gshift, gscale, B, p.nchunk, 2, C, p.mbf, s);
@@ -857,9 +855,8 @@ int dmf_gate_residual_fwd(const void* x, const void* tx, const void* gate, const
   p.xbf = x_dtype == DMF_ATTN_BF16; p.mbf = mod_dtype == DMF_ATTN_BF16; p.hbf = h_dtype == DMF_ATTN_BF16;
   const unsigned grid = static_cast<unsigned>((p.total + kThreads - 1) / kThreads);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (ty) hipLaunchKernelGGL(gate_residual_fwd_kernel<true>, dim3(grid), dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL(gate_residual_fwd_kernel<false>, dim3(grid), dim3(kThreads), 0, s, p);
-  return launch_status();
+  if (ty) return launch_kernel(gate_residual_fwd_kernel<true>, dim3(grid), dim3(kThreads), 0, s, p);
+  return launch_kernel(gate_residual_fwd_kernel<false>, dim3(grid), dim3(kThreads), 0, s, p);
 }
 
 int dmf_gate_residual_bwd(const void* gy, const void* gate, const void* h, void* gh, void* ggate, float* workspace,
@@ -880,7 +877,7 @@ int dmf_gate_residual_bwd(const void* gy, const void* gate, const void* h, void*
   const int rc = dispatch_nv(C, [&](auto nv) {
     constexpr int NV = decltype(nv)::value;
     constexpr size_t lds = (kWaves - 1) * NV * 512 * sizeof(float);
-    hipLaunchKernelGGL((gate_residual_bwd_kernel<NV>), dim3(grid), dim3(kThreads), lds, s, p);
+    return launch_kernel(gate_residual_bwd_kernel<NV>, dim3(grid), dim3(kThreads), lds, s, p);
   });
   if (rc) return rc;
   return reduce_partials(workspace, ggate, nullptr, B, p.nchunk, 1, C, p.mbf, s);
@@ -916,8 +913,8 @@ int dmf_residual_ln_modulate_fwd(const void* x, const void* tx, const void* gate
   hipStream_t s = static_cast<hipStream_t>(stream);
   return dispatch_nv(C, [&](auto nv) {
     constexpr int NV = decltype(nv)::value;
-    if (jvp) hipLaunchKernelGGL((residual_ln_modulate_fwd_kernel<NV, true>), dim3(grid), dim3(kThreads), 0, s, p);
-    else hipLaunchKernelGGL((residual_ln_modulate_fwd_kernel<NV, false>), dim3(grid), dim3(kThreads), 0, s, p);
+    if (jvp) return launch_kernel(residual_ln_modulate_fwd_kernel<NV, true>, dim3(grid), dim3(kThreads), 0, s, p);
+    return launch_kernel(residual_ln_modulate_fwd_kernel<NV, false>, dim3(grid), dim3(kThreads), 0, s, p);
   });
 }
 
@@ -952,8 +949,7 @@ int dmf_colsum(const void* x, void* out, float* workspace, int64_t rows, int C, 
   p.x = x; p.partial = workspace; p.rows = rows; p.C = C; p.xbf = x_dtype == DMF_ATTN_BF16;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(nchunk), static_cast<unsigned>((C / 8 + 63) / 64));
-  hipLaunchKernelGGL(colsum_kernel, grid, dim3(kThreads), 0, s, p);
-  if (int rc = launch_status()) return rc;
+  if (int rc = launch_kernel(colsum_kernel, grid, dim3(kThreads), 0, s, p)) return rc;
   return reduce_partials(workspace, out, nullptr, 1, static_cast<int>(nchunk), 1, C, out_dtype == DMF_ATTN_BF16, s);
 }
 
@@ -991,9 +987,8 @@ int dmf_rmsnorm_fwd(const void* x, const void* tx, const void* gain, void* y, vo
   p.bf = dtype == DMF_ATTN_BF16; p.gbf = gain_dtype == DMF_ATTN_BF16;
   const unsigned grid = static_cast<unsigned>((p.rows + kThreads / 16 - 1) / (kThreads / 16));
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (ty) hipLaunchKernelGGL(rmsnorm_fwd_kernel<true>, dim3(grid), dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL(rmsnorm_fwd_kernel<false>, dim3(grid), dim3(kThreads), 0, s, p);
-  return launch_status();
+  if (ty) return launch_kernel(rmsnorm_fwd_kernel<true>, dim3(grid), dim3(kThreads), 0, s, p);
+  return launch_kernel(rmsnorm_fwd_kernel<false>, dim3(grid), dim3(kThreads), 0, s, p);
 }
 
 int dmf_rmsnorm_bwd(const void* gy, const void* x, const void* gain, void* gx, void* ggain, float* workspace,
@@ -1012,8 +1007,7 @@ int dmf_rmsnorm_bwd(const void* gy, const void* x, const void* gain, void* gx, v
   const int64_t want = (p.rows + kThreads / 16 - 1) / (kThreads / 16);
   const int nblocks = static_cast<int>(std::min<int64_t>(want, kRmsBlocksMax));
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(rmsnorm_bwd_kernel, dim3(nblocks), dim3(kThreads), 0, s, p);
-  if (int rc = launch_status()) return rc;
+  if (int rc = launch_kernel(rmsnorm_bwd_kernel, dim3(nblocks), dim3(kThreads), 0, s, p)) return rc;
   return reduce_partials(workspace, ggain, nullptr, 1, nblocks, 1, D, p.gbf, s);
 }
 

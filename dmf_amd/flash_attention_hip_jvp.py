@@ -183,6 +183,8 @@ def flash_attn_func(q, k, v, softmax_scale=None):
             tangents.append(torch.zeros_like(p) if tg is None else tg)
         out, _, t_out = _lib.run_function(FlashAttnFunc, *primals, *tangents, softmax_scale)
         return fwAD.make_dual(out, t_out)
+    if _lib.plain_inference(q, k, v):
+        return _lib.fwd(q, k, v, _default_scale(q, softmax_scale), need_lse=False)[0]
     out, _, _ = _lib.run_function(FlashAttnFunc, q, k, v, None, None, None, softmax_scale)
     return out
 
@@ -241,6 +243,9 @@ def flash_attn_qkvpacked_func(qkv, softmax_scale=None):
     if qkv.dim() != 5 or qkv.shape[2] != 3:
         raise ValueError(f"expected a packed (B, L, 3, H, D) tensor, got shape {tuple(qkv.shape)}")
     p, tg = fwAD.unpack_dual(qkv)
+    if tg is None and _lib.plain_inference(p):
+        q, k, v = p.unbind(2)
+        return _lib.fwd(q, k, v, _default_scale(q, softmax_scale), need_lse=False)[0]
     out, _, t_out = _lib.run_function(FlashAttnQKVPackedFunc, p, tg, softmax_scale)
     return out if tg is None else fwAD.make_dual(out, t_out)
 
@@ -314,5 +319,14 @@ def flash_attn_qknorm_qkvpacked_func(qkv, q_gain, k_gain, eps: float = 1e-6, sof
     if qkv.dim() != 5 or qkv.shape[2] != 3:
         raise ValueError(f"expected a packed (B, L, 3, H, D) tensor, got shape {tuple(qkv.shape)}")
     p, tg = fwAD.unpack_dual(qkv)
+    if tg is None and _lib.plain_inference(p, q_gain, k_gain):
+        q, k, v = p.unbind(2)
+        scale = _default_scale(q, softmax_scale)
+        kn, _ = _lib.rmsnorm_fwd(k, k_gain, None, eps, False)
+        fused = _lib.fwd_qnorm(q, kn, v, None, None, None, q_gain, eps, scale, need_lse=False) if IN_KERNEL_Q_NORM else None
+        if fused is not None:
+            return fused[0]
+        qn, _ = _lib.rmsnorm_fwd(q, q_gain, None, eps, False)
+        return _lib.fwd(qn, kn, v, scale, need_lse=False)[0]
     out, _, t_out, _, _ = _lib.run_function(QKNormAttnQKVPackedFunc, p, tg, q_gain, k_gain, eps, softmax_scale)
     return out if tg is None else fwAD.make_dual(out, t_out)

@@ -159,22 +159,25 @@ def fm_loss(model, x, y, t, eps, path_type: str = "linear"):
     return loss, {"fm_loss": fm}
 
 
-def dmf_train_step(model, batch, model_t=None, functorch: bool = True, **guidance):
+def dmf_train_step(model, batch, model_t=None, functorch: bool = True, autocast: bool = True, **guidance):
     """One optimisation step's forward and backward as train_dmf.py:325-330 runs
     them: ``dmf_loss`` under bf16 autocast, mean over the batch, backward.  The
     parameters do not change between the (up to four) model calls of one step, so
     the fused Linear layers share one bf16 copy of their weights per step instead
     of casting them in every call; gradients still reach the fp32 parameters."""
-    with frozen_low_precision_params(model), torch.autocast("cuda", dtype=torch.bfloat16):
+    with contextlib.ExitStack() as stack:
+        if autocast:   # (``autocast=False``: the same step in the parameters' own precision, e.g. an fp32 yardstick)
+            stack.enter_context(frozen_low_precision_params(model))
+            stack.enter_context(torch.autocast("cuda", dtype=torch.bfloat16))
         loss, _ = dmf_loss(model, *batch, model_t=model_t, functorch=functorch, **guidance)
         loss = loss.mean()
         loss.backward()
     return loss
 
 
-def fm_train_step(model, batch):
+def fm_train_step(model, batch, autocast: bool = True):
     """train_fm.py:347-352: ``fm_loss`` under bf16 autocast, mean, backward."""
-    with torch.autocast("cuda", dtype=torch.bfloat16):
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
         loss, _ = fm_loss(model, *batch)
     loss = loss.mean()
     loss.backward()

@@ -9,6 +9,7 @@ import torch
 from dmf_amd import harness
 from dmf_amd.dmft import DMFT, DMFT_models
 from oracle import attn_oracle as ao
+from parity_util import grads, no_worse_than_base
 
 
 def _small(attn_func, **kw):
@@ -208,6 +209,60 @@ def test_dmft_b2_full_architecture_fused_graph_vs_base():
         u, du = graphed(*data)
         assert ao.rel_l2(u.float().cpu(), u_ref.float().cpu()) <= 3e-2
         assert ao.rel_l2(du.float().cpu(), du_ref.float().cpu()) <= 3e-2
+
+
+@pytest.mark.gpu
+def test_dmft_xl2_config5_train_step_fused_and_graph_vs_base():
+    """The full DMFT-XL/2 256px training step at its real architecture (models/dmft.py:170: 28 blocks, hidden 1152,
+    16 heads of 72, 256 tokens; dmf_depth 20), random trunc-normal weights, reduced batch: forward + JVP through the new
+    attention and the fused block glue, then backward on the primal output with the JVP target detached
+    (loss.py:165-173, train_dmf.py:320-335), eagerly and replayed as a HIP graph.  Yardstick: the same weights and
+    inputs through the naive attention and the reference's expressions in fp32; the bf16-autocast reference path
+    measures how far rounding alone moves u, du/dt, the loss and every parameter gradient, and the fused path may
+    move them at most 1.5 times as far."""
+    dev = "cuda:0"
+    m_ref = harness.build_model("DMFT-XL/2", "base", dev, dmf_depth=20)
+    assert (len(m_ref.blocks), m_ref.num_heads, m_ref.pos_embed.shape, m_ref.dmf_depth) == (28, 16, (1, 256, 1152), 20)
+    data = harness.synthetic_batch(2, dev)
+
+    def run(model, autocast):
+        model.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            loss, u, du = harness.meanflow_loss(model, *data)
+        loss.backward()
+        return float(loss), u.detach().float().cpu(), du.detach().float().cpu(), grads(model)
+
+    l32, u32, du32, g32 = run(m_ref, False)
+    lb, ub, dub, gb = run(m_ref, True)
+    m = harness.build_model("DMFT-XL/2", "hip", dev, dmf_depth=20, block_ops="hip")
+    m.load_state_dict(m_ref.state_dict())
+    del m_ref
+    lf, uf, duf, gf = run(m, True)
+    eu, edu = ao.rel_l2(ub, u32), ao.rel_l2(dub, du32)
+    print(f"base-bf16 vs fp32: u {eu:.3e} du {edu:.3e} loss {abs(lb - l32) / abs(l32):.3e}; "
+          f"fused: u {ao.rel_l2(uf, u32):.3e} du {ao.rel_l2(duf, du32):.3e} loss {abs(lf - l32) / abs(l32):.3e}", flush=True)
+    assert ao.rel_l2(uf, u32) <= 1.5 * eu + 2e-3 and ao.rel_l2(duf, du32) <= 1.5 * edu + 2e-3
+    assert abs(lf - l32) <= 1.5 * abs(lb - l32) + 2e-3 * abs(l32)
+    no_worse_than_base(gf, gb, g32)
+    del gb, g32
+
+    # the same step captured once and replayed: same loss and gradients as the eager fused step, to rounding
+    def step(*b):
+        m.zero_grad(set_to_none=True)
+        return harness.train_step(m, b, functorch=False).detach()
+
+    m.zero_grad(set_to_none=True)
+    eager_loss = float(step(*data))
+    eager = grads(m)
+    m.zero_grad(set_to_none=True)
+    graphed = harness.GraphedStep(step, *data)
+    for _ in range(2):
+        out = graphed(*data)
+        torch.cuda.synchronize()
+        assert abs(float(out) - eager_loss) <= 1e-3 * abs(eager_loss)
+        got = grads(m)
+        worst = max((ao.rel_l2(got[n], eager[n]), n) for n in eager if float(eager[n].abs().max()) > 0)
+        assert worst[0] <= 2e-3, worst
 
 
 @pytest.mark.gpu
