@@ -47,6 +47,7 @@ SIGNATURES = {
     "dmf_rmsnorm_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_rmsnorm_bwd": (c_int, [_P] * 6 + [_S] + [_I] * 4 + [_F, _I, _I, _P]),
     "dmf_colsum": (c_int, [_P] * 3 + [_L, _I, _I, _I, _P]),
+    "dmf_colsum_static": (c_int, [_P] * 2 + [_L, _I, _I, _I, _P]),
     "dmf_residual_ln_modulate_fwd": (c_int, [_P] * 14 + [_S] + [_I] * 3 + [_F] + [_I] * 4 + [_P]),
     "dmf_silu_fwd": (c_int, [_P] * 4 + [_L, _I, _I, _P]),
     "dmf_silu_bwd": (c_int, [_P] * 3 + [_L, _I, _I, _P]),

@@ -953,6 +953,38 @@ int dmf_colsum(const void* x, void* out, float* workspace, int64_t rows, int C, 
   return reduce_partials(workspace, out, nullptr, 1, static_cast<int>(nchunk), 1, C, out_dtype == DMF_ATTN_BF16, s);
 }
 
+// ---- dmf_colsum for callers that cannot allocate: the partial sums live in library-owned device memory -------------
+//
+// `colsum_scratch` is the name of a per-device symbol, not a device address: host code may only use the address that
+// hipGetSymbolAddress returns for the current device (each GPU holds its own copy of the array at its own address).
+constexpr int64_t kColsumStaticFloats = DMF_COLSUM_STATIC_MAX_FLOATS;
+static __device__ __align__(256) float colsum_scratch[kColsumStaticFloats];
+
+// Address of this device's copy of the array, looked up once per device (a race between two host threads at worst
+// repeats the idempotent lookup).  Returns nullptr if the runtime cannot resolve the symbol.
+static float* colsum_scratch_on_current_device() {
+  static float* addr[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  if (addr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(colsum_scratch)) != hipSuccess) return nullptr;
+    addr[dev] = static_cast<float*>(p);
+  }
+  return addr[dev];
+}
+
+int dmf_colsum_static(const void* x, void* out, int64_t rows, int C, int x_dtype, int out_dtype, void* stream) {
+  // size check first, so that an oversized request is refused whatever else is wrong with it
+  if (rows < 1 || C < 8 || C % 8) return DMF_ATTN_ESHAPE;
+  const int64_t nchunk = (rows + kColsumRows - 1) / kColsumRows;
+  if (nchunk > kColsumStaticFloats / C) return DMF_ATTN_ESCRATCH;
+  float* ws = colsum_scratch_on_current_device();
+  if (ws == nullptr) return DMF_ATTN_ELAUNCH;
+  // Stage one overwrites every partial sum that stage two reads, so nothing has to be cleared between calls.
+  return dmf_colsum(x, out, ws, rows, C, x_dtype, out_dtype, stream);
+}
+
 // Validates a strided (B, L, H, D) operand and copies {sB, sL, sH}.
 static int check_blhd(const void* ptr, const int64_t* st4, int eb, int64_t (&st3)[3]) {
   if (!aligned16(ptr)) return DMF_ATTN_EALIGN;

@@ -48,6 +48,7 @@ const char* dmf_attn_strerror(int code) {
     case DMF_ATTN_EALIGN: return "a base pointer is not 16-byte aligned";
     case DMF_ATTN_ELAUNCH: return "the HIP runtime rejected the kernel launch";
     case DMF_ATTN_ENOKERNEL: return "no kernel implements this variant for the given shape / dtype";
+    case DMF_ATTN_ESCRATCH: return "the problem needs more scratch memory than the library's static buffer holds (use the entry point that takes a workspace)";
     default: return "unknown error code";
   }
 }

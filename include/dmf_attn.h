@@ -58,7 +58,8 @@ enum {
   DMF_ATTN_ENULL = -5,     /* a required pointer is NULL                        */
   DMF_ATTN_EALIGN = -6,    /* a base pointer is not 16-byte aligned             */
   DMF_ATTN_ELAUNCH = -7,   /* the HIP runtime rejected the launch               */
-  DMF_ATTN_ENOKERNEL = -8  /* no kernel implements this variant for the given shape / dtype; nothing was launched */
+  DMF_ATTN_ENOKERNEL = -8, /* no kernel implements this variant for the given shape / dtype; nothing was launched */
+  DMF_ATTN_ESCRATCH = -9   /* the problem needs more scratch memory than the library's static buffer holds        */
 };
 
 /* Library version, (major << 16) | minor. */

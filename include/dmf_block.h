@@ -173,6 +173,28 @@ DMF_ATTN_API int dmf_rmsnorm_bwd(const void* gy, const void* x, const void* gain
 DMF_ATTN_API int dmf_colsum(const void* x, void* out, float* workspace, int64_t rows, int C, int x_dtype,
                             int out_dtype, void* stream);
 
+/*
+ * dmf_colsum without a workspace argument and without any allocation: the
+ * partial sums of the first stage are kept in a file-scope device array inside
+ * the library (DMF_COLSUM_STATIC_MAX_FLOATS fp32 values = 4 MiB, held by every
+ * GPU the library runs on until the process ends).  This entry point has no
+ * counterpart in the reference; it exists for callers that cannot allocate --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc -- and calls no hipMalloc / hipFree or allocating library routine.
+ * Same kernels and the same bits as dmf_colsum.
+ *   - Limit: ceil(rows / 64) * C <= DMF_COLSUM_STATIC_MAX_FLOATS, otherwise
+ *     DMF_ATTN_ESCRATCH is returned and nothing is launched (e.g. 8192 x 4608
+ *     or 32768 x 1152 fit; use dmf_colsum with your own workspace beyond).
+ *   - All calls on one GPU share that GPU's array: two calls that overlap in
+ *     time on the same GPU (different streams, or host threads launching
+ *     concurrently) race on it.  Calls ordered on one stream are safe, and
+ *     nothing needs clearing between them (every partial sum a call reads was
+ *     written by that call).
+ */
+#define DMF_COLSUM_STATIC_MAX_FLOATS (1 << 20)
+DMF_ATTN_API int dmf_colsum_static(const void* x, void* out, int64_t rows, int C, int x_dtype, int out_dtype,
+                                   void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,12 +29,12 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = _declared_symbols()
-    assert len(names) == 19 and set(names) == set(_lib.SIGNATURES), names
+    assert len(names) == 20 and set(names) == set(_lib.SIGNATURES), names
     for n in names:
         assert getattr(lib, n) is not None
     assert lib.dmf_attn_version() >= 1
     assert lib.dmf_attn_strerror(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-9, 0):
         assert b"unknown" not in lib.dmf_attn_strerror(code)
     assert b"unknown" in lib.dmf_attn_strerror(-99)
 
