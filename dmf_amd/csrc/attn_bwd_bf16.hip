@@ -11,6 +11,10 @@
 #include "attn_kernels.h"
 #include <algorithm>
 
+#ifndef DMF_BWD_FUSED
+#define DMF_BWD_FUSED 1   // 0: two kernels always; 1: single-pass kernel for 128 < max(Lq, Lkv) <= 256; 2: for every length <= 256
+#endif
+
 namespace dmf {
 
 template <int D>
@@ -352,6 +356,396 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
                                       });
 }
 
+// 8-byte LDS store issued as a raw instruction, for the same reason as the untracked reads in attn_common.h (a store
+// the compiler knows about would be preceded by a full vmcnt(0) while a tile DMA is in flight).  The data is in LDS
+// once a later `s_waitcnt lgkmcnt(0)` of this wave has passed (LDS operations complete in order).
+template <int OFF>
+__device__ __forceinline__ void lds_write64_untracked(uint32_t addr, u32x2 w) {
+  asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(addr), "v"(w), "n"(OFF) : "memory");
+}
+
+template <int OFF>
+__device__ __forceinline__ void lds_write128_untracked(uint32_t addr, u32x4 w) {
+  asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(w), "n"(OFF) : "memory");
+}
+
+// ------------------------------------------------ single-pass backward, whole (batch, head) unit per work-group
+// For sequences of at most 256 rows one 8-wave work-group owns a whole (batch, head) unit and every score tile is
+// formed exactly once -- 5 GEMM units per (query tile, key tile) pair instead of the 7 of the two-kernel scheme --
+// with no atomics, no workspace and a fixed summation order:
+//   * wave w owns keys 32w .. 32w+31: K (times scale*log2e) and V stay in registers as B operands, dK^T and dV^T are
+//     its accumulators over the whole sequence ("phase 1", the dK/dV kernel's loop body: S = Q K^T, dP = dout V^T,
+//     P, dS, dV^T += dout^T P, dK^T += Q^T dS, with Q / dout tiles of 32 queries streamed HBM -> LDS by DMA);
+//   * dQ needs dS contracted over keys, i.e. across the waves.  Instead of summing eight fp32 partial tiles, the bf16
+//     dS tiles themselves are exchanged: phase 1 leaves tile (query tile j, key block w) in an LDS array X, and after
+//     four query tiles ("half" of the sequence; 64 KB of X) "phase 2" forms dQ^T = K^T dS^T for those 128 queries from X
+//     and an LDS-resident copy of K.  The 3 (head dim 72: 2 + remainder) output tiles of a query tile are split
+//     between wave jj (tiles of part 0) and wave jj + 4 (part 1) -- two waves of the same SIMD, so every SIMD gets the
+//     same MFMA work and no partial sums have to be combined.
+// LDS: K (8 tiles) | NST stages of Q, dout tiles | X (64 KB, reused as store staging) | lse, delta of all rows.
+template <int D>
+struct BwdFusedCfg {
+  using F = BwdFastCfg<D>;
+  static constexpr int TB = F::TBYTES;
+  static constexpr int XBYTES = 65536, STATBYTES = 2 * 256 * 4;
+  // Q / dout stages: as many as the LDS has room for (4: tiles are requested three iterations ahead, which covers the
+  // HBM latency of a work-group that has the CU to itself)
+  static constexpr int NST = (8 + 2 * 4) * TB + XBYTES + STATBYTES <= 160 * 1024 ? 4 : ((8 + 2 * 3) * TB + XBYTES + STATBYTES <= 160 * 1024 ? 3 : 2);
+  static constexpr int K_OFF = 0, QS_OFF = 8 * TB, X_OFF = QS_OFF + 2 * NST * TB, STAT_OFF = X_OFF + XBYTES;
+  static constexpr int LDS_BYTES = STAT_OFF + STATBYTES;
+  static constexpr int XTILE = 32 * 32 * 2;                      // one exchanged dS tile: [32 keys][32 queries] bf16
+  static constexpr int NT0 = (F::NMT + 1) / 2;                   // part 0: output tiles 0 .. NT0-1 (+ the 16-wide remainder); part 1: the rest
+  static_assert(LDS_BYTES <= 160 * 1024, "head dim too large for the single-pass backward");
+  static_assert(256 * Cfg<__bf16, D>::OROWV * 16 <= XBYTES, "store staging must fit the exchange area");
+};
+
+template <int D>
+__global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdParams p) {
+  using F = BwdFastCfg<D>;
+  using FC = BwdFusedCfg<D>;
+  using T = __bf16;
+  constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR, TB = FC::TB;
+  constexpr bool TAIL = F::TAIL;
+  constexpr int DO_OFF = TB;               // dout tile sits after the Q tile of its stage
+  constexpr int STAGE = 2 * TB;
+  constexpr int NT0 = FC::NT0, NST = FC::NST;
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, g = lane >> 5;
+  const int bh = xcd_remap(blockIdx.x, gridDim.x);
+  const int b = bh / p.H, h = bh % p.H;
+  auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
+  float* stat_lse = reinterpret_cast<float*>(smem + FC::STAT_OFF);
+  float* stat_delta = stat_lse + 256;
+
+  // ---- zero the contraction padding of the K tiles and of both Q / dout stages
+  if constexpr (P > VPR) {
+    constexpr int PADV = P - VPR;
+    for (int i = tid; i < (8 + 2 * NST) * 32 * PADV; i += 512) {
+      const int tile = i / (32 * PADV), r = (i / PADV) % 32, cv = VPR + i % PADV;
+      *reinterpret_cast<u32x4*>(smem + tile * TB + (r * P + cv) * 16) = u32x4{0, 0, 0, 0};
+    }
+  }
+
+  const uint32_t rb_q = (uint32_t)p.st[1][1] * 2, rb_do = (uint32_t)p.st[0][1] * 2;
+  const uint32_t rb_k = (uint32_t)p.st[2][1] * 2, rb_v = (uint32_t)p.st[3][1] * 2;
+  const __amdgpu_buffer_rsrc_t rs_q = make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(1), rb_q, p.Lq, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_do = make_rows_rsrc(reinterpret_cast<const T*>(p.dout) + base(0), rb_do, p.Lq, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_k = make_rows_rsrc(reinterpret_cast<const T*>(p.k) + base(2), rb_k, p.Lkv, D * 2);
+  const __amdgpu_buffer_rsrc_t rs_v = make_rows_rsrc(reinterpret_cast<const T*>(p.v) + base(3), rb_v, p.Lkv, D * 2);
+  const int nqt = (p.Lq + 31) / 32, nkb = (p.Lkv + 31) / 32;   // query tiles / key blocks in use (<= 8 each)
+
+  // ---- requests, in the order in which their data is needed (a work-group has its CU to itself, so whatever the
+  //      first tile waits for is exposed; the memory system serves the requests roughly first come, first served):
+  //      lse and the first tile's dout / o rows (for delta), the first Q / dout tile, this wave's K and V rows, further
+  //      tiles.
+  // Every wave issues exactly two DMA instructions per Q / dout tile, and
+  // wait_tile(j) lets the ones issued after tile j stay in flight (vector memory operations complete in order, and
+  // anything not counted here can only make the wait stricter).
+  // Tiles 0 .. NST-2 are requested up front, then tile j+NST-1 at the top of iteration j: when tile j is waited for,
+  // the tiles j+1 .. j+NST-2 (as far as they exist) were requested after it.
+  auto issue_q = [&](int j) {   // tile j goes to stage j % NST
+    char* st = smem + FC::QS_OFF + (j % NST) * STAGE;
+    issue_tile_rows<P, VPR, 8>(rs_q, rb_q, (uint32_t)j * 32 * rb_q, st, wave, lane);
+    issue_tile_rows<P, VPR, 8>(rs_do, rb_do, (uint32_t)j * 32 * rb_do, st + DO_OFF, wave, lane);
+  };
+  auto wait_tile = [&](int j) {
+    const int newer = 2 * min(NST - 2, nqt - 1 - j);
+    if (newer >= 12) __builtin_amdgcn_s_waitcnt(0x0F7C);
+    else if (newer >= 8) __builtin_amdgcn_s_waitcnt(0x0F78);
+    else if (newer >= 4) __builtin_amdgcn_s_waitcnt(0x0F74);
+    else if (newer >= 2) __builtin_amdgcn_s_waitcnt(0x0F72);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+  };
+  // delta = rowsum(dout * o) of the 32 query rows of a tile, by the whole work-group: 16 lanes per row, one 16-byte
+  // vector of dout and of o per lane (lanes past the head dim read zeros), summed across the 16 lanes.
+  const uint32_t rb_o = (uint32_t)p.st[4][1] * 2;
+  const __amdgpu_buffer_rsrc_t rs_o = make_rows_rsrc(reinterpret_cast<const T*>(p.o) + base(4), rb_o, p.Lq, D * 2);
+  struct DeltaRows { u32x4 d, o; };
+  auto delta_request = [&](int j) {
+    const int qrow = 32 * j + (tid >> 4), cv = tid & 15;
+    DeltaRows r;
+    r.d = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_do, cv < VPR ? (uint32_t)qrow * rb_do + cv * 16 : 0x7ffffff0u, 0, 0));
+    r.o = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_o, cv < VPR ? (uint32_t)qrow * rb_o + cv * 16 : 0x7ffffff0u, 0, 0));
+    return r;
+  };
+  auto delta_finish = [&](int j, const DeltaRows& r) {
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s += __uint_as_float(r.d[e] << 16) * __uint_as_float(r.o[e] << 16);
+      s += __uint_as_float(r.d[e] & 0xffff0000u) * __uint_as_float(r.o[e] & 0xffff0000u);
+    }
+    // inclusive sum over the row of 16 lanes (DPP row_shr 1, 2, 4, 8; lanes shifted in from outside read 0): lane 15 holds it
+    auto shr = [](float x, auto n) {
+      return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x110 + decltype(n)::value, 0xf, 0xf, true));
+    };
+    s += shr(s, std::integral_constant<int, 1>{});
+    s += shr(s, std::integral_constant<int, 2>{});
+    s += shr(s, std::integral_constant<int, 4>{});
+    s += shr(s, std::integral_constant<int, 8>{});
+    const int qrow = 32 * j + (tid >> 4);
+    if ((tid & 15) == 15) {
+      const bool qok = qrow < p.Lq;
+      stat_delta[qrow] = qok ? s : 0.f;
+      if (qok) p.delta[(int64_t)bh * p.Lq + qrow] = s;
+    }
+  };
+
+  if (tid < 256) stat_lse[tid] = tid < p.Lq ? p.lse[(int64_t)bh * p.Lq + tid] : INFINITY;   // +inf switches padded query rows off (P = 0)
+  DeltaRows dr = delta_request(0);
+  issue_q(0);
+  // ---- this lane's key row: K (times scale*log2e) and V stay in registers
+  const int krow = wave * 32 + c32;
+  u32x4 Kr[NCHUNK], Vr[NCHUNK];
+  load_row_chunks<NCHUNK, VPR>(rs_k, rb_k, krow, g, Kr);
+  load_row_chunks<NCHUNK, VPR>(rs_v, rb_v, krow, g, Vr);
+  for (int j = 1; j < NST - 1 && j < nqt; ++j) issue_q(j);
+  // the LDS-resident copy of K (phase 2 operand) comes from these registers rather than from a second trip to memory:
+  // lane (c32, g) holds vectors 2c + g of row krow (rows past Lkv were read as zeros)
+  {
+    const uint32_t ka = lds_addr(smem) + FC::K_OFF + (krow * P + g) * 16;
+    static_for<NCHUNK>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      if (2 * c + g < VPR) lds_write128_untracked<32 * c>(ka, Kr[c]);
+    });
+  }
+  delta_finish(0, dr);
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) Kr[c] = scale_bf16x8(Kr[c], p.scale_log2);
+  const bool kvalid = krow < p.Lkv;
+
+  f32x16 dK[NMT], dV[NMT];
+  f32x4 dK16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}}, dV16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+#pragma unroll
+  for (int t = 0; t < NMT; ++t) {
+    dK[t] = f32x16{0};
+    dV[t] = f32x16{0};
+  }
+
+  // lane addresses (relative to a tile base): row-operand reads, transposed reads, remainder operand
+  const uint32_t row_addr = lds_addr(smem) + c32 * STR * 2 + g * 16;
+  const uint32_t col_off = ((4 * g + ((lane & 15) >> 2)) * STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const uint32_t tail_off = tail_lane_offset(lane, STR, 32 * NMT) * 2;
+  // exchange tiles: [32 keys][32 queries] bf16, pitch 64 bytes
+  const uint32_t x_base = lds_addr(smem) + FC::X_OFF;
+  // The eight 8-byte pieces (4 queries) of key row k are stored at piece index (piece ^ ((k >> 2) & 7)): without the
+  // swizzle the 64 lanes of a store (key = lane % 32, row pitch 64 bytes) fall on 8 of the 32 bank pairs.
+  const uint32_t x_swz = (c32 >> 2) & 7;
+
+  for (int half = 0; half * 4 < nqt; ++half) {
+    // ================= phase 1: query tiles 4*half .. 4*half+3 against this wave's keys
+    const int j_end = min(nqt, 4 * half + 4);
+    for (int j = 4 * half; j < j_end; ++j) {
+      if (j == 0 || j != 4 * half) {   // (the first tile of a later half was waited for before the dQ rows were stored)
+        wait_tile(j);     // this wave's share of tile j has landed
+        if (j == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and its rows of the K copy are in LDS
+        lds_barrier();    // ... and everyone else's; all waves are done with the stage of tile j-1
+      }
+      if (j + 1 < nqt) dr = delta_request(j + 1);   // (before the tile request: its data is wanted first)
+      if (j + NST - 1 < nqt) issue_q(j + NST - 1);
+      const uint32_t stage_off = FC::QS_OFF + (j % NST) * STAGE;
+      const uint32_t ra = row_addr + stage_off, ca = lds_addr(smem) + col_off + stage_off;
+
+      // ---- S = Q K^T (log2 units), dP = dout V^T : rows = queries (in-lane), columns = keys (lanes)
+      f32x16 S = {0}, dP = {0};
+      {
+        u32x4 qc[2], oc[2];
+        qc[0] = lds_read128_issue<0>(ra);
+        oc[0] = lds_read128_issue<DO_OFF>(ra);
+        static_for<NCHUNK>([&](auto cc) {
+          constexpr int c = decltype(cc)::value;
+          constexpr bool more = c + 1 < NCHUNK;
+          if constexpr (more) {
+            qc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
+            oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
+          }
+          lds_read128_wait<more ? 2 : 0>(qc[c & 1], oc[c & 1]);
+          mma_chunk<T>(S, qc[c & 1], Kr[c]);
+          mma_chunk<T>(dP, oc[c & 1], Vr[c]);
+        });
+      }
+      // ---- P = exp2(S - lse*log2e), dS = P * (dP - delta); padded query rows carry lse = +inf (P = 0), padded keys are
+      //      switched off below
+      f32x16 Pm, dS;
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(stat_lse + j * 32 + jj * 8 + 4 * g);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(stat_delta + j * 32 + jj * 8 + 4 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * jj + e;
+          Pm[i] = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
+          dS[i] = Pm[i] * (dP[i] - d4[e]);
+        }
+      }
+      ColOperand pp[2] = {acc_operand<T>(Pm, 0), acc_operand<T>(Pm, 1)};
+      ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
+      // ---- dS tile -> X[j % 4][wave] (zeros for keys past the end: their K rows must not reach dQ)
+      {
+        const uint32_t xa = x_base + ((j & 3) * 8 + wave) * FC::XTILE + c32 * 64;
+        static_for<4>([&](auto jc) {
+          constexpr int jj = decltype(jc)::value;
+          const u32x2 w = kvalid ? u32x2{ds[jj >> 1].v[2 * (jj & 1)], ds[jj >> 1].v[2 * (jj & 1) + 1]} : u32x2{0, 0};
+          lds_write64_untracked<0>(xa + (((2 * jj + g) ^ x_swz) << 3), w);   // queries 8jj + 4g .. +3 of key row c32
+        });
+      }
+      // ---- dV^T += dout^T P ; dK^T += Q^T dS
+      {
+        constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
+        TrPair qq[2], oo[2];
+        auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
+        qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
+        oo[0] = lds_tr16_issue<lo_off(0) + DO_OFF, lo_off(0) + 8 * STR * 2 + DO_OFF>(ca);
+        static_for<NGT>([&](auto gc) {
+          constexpr int gi = decltype(gc)::value;
+          constexpr bool more = gi + 1 < NGT;
+          if constexpr (gi + 1 < NG) {
+            constexpr int LO = lo_off(gi + 1), HI = LO + 8 * STR * 2;
+            qq[(gi + 1) & 1] = lds_tr16_issue<LO, HI>(ca);
+            oo[(gi + 1) & 1] = lds_tr16_issue<LO + DO_OFF, HI + DO_OFF>(ca);
+          } else if constexpr (more) {
+            const uint32_t ta = lds_addr(smem) + tail_off + stage_off;
+            qq[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(ta);
+            oo[(gi + 1) & 1] = lds_tr16_issue<DO_OFF, 8 * STR * 2 + DO_OFF>(ta);
+          }
+          lds_tr16_wait<more ? 4 : 0>(qq[gi & 1], oo[gi & 1]);
+          if constexpr (gi < NG) {
+            mma_col<T>(dV[gi % NMT], tr_operand(oo[gi & 1]), pp[gi / NMT]);
+            mma_col<T>(dK[gi % NMT], tr_operand(qq[gi & 1]), ds[gi / NMT]);
+          } else {
+            ColOperand p0, p1, d0, d1;
+            tail_operands(pp[0], pp[1], p0, p1);
+            tail_operands(ds[0], ds[1], d0, d1);
+            mma16(dV16[0], tr_operand(oo[gi & 1]), p0);
+            mma16(dV16[1], tr_operand(oo[gi & 1]), p1);
+            mma16(dK16[0], tr_operand(qq[gi & 1]), d0);
+            mma16(dK16[1], tr_operand(qq[gi & 1]), d1);
+          }
+        });
+      }
+      if (j + 1 < nqt) delta_finish(j + 1, dr);   // visible to the other waves after the next barrier
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's dS tiles are in LDS
+    lds_barrier();                                        // X holds every dS tile of this half
+
+    // ================= phase 2: dQ^T = K^T dS^T for query tile jq, output tiles of this wave's part
+    const int jq = 4 * half + (wave & 3);
+    const bool part1 = wave >= 4;
+    f32x16 dQ[NT0];
+    f32x4 dQ16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+#pragma unroll
+    for (int t = 0; t < NT0; ++t) dQ[t] = f32x16{0};
+    if (jq < nqt) {
+      // Operands through the tracked LDS-read intrinsics here, not the raw-instruction helpers of phase 1: those are
+      // only safe in straight-line code (between the issue and the wait the compiler may copy the destination
+      // registers, e.g. at a branch, and would copy stale data), and this loop branches on the wave's part.  The
+      // price is that the compiler waits for the tile DMA in flight before the first read, which was requested a
+      // whole tile earlier.
+      const T* xt = reinterpret_cast<const T*>(smem + FC::X_OFF) + (wave & 3) * 8 * (FC::XTILE / 2);
+      // lds_col_operand on a swizzled exchange tile: key rows 16s + 4g + (i >> 2) (+ 8), query piece 4 * half + (i & 3)
+      auto x_operand = [&](const T* tile, int st) {
+        const int i = lane & 15, piece = 4 * ((lane >> 4) & 1) + (i & 3), r = 16 * st + 4 * g + (i >> 2);
+        const T* lo = tile + r * 32 + ((piece ^ ((r >> 2) & 7)) << 2);
+        const T* hi = tile + (r + 8) * 32 + ((piece ^ (((r + 8) >> 2) & 7)) << 2);
+        const u32x2 a = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, lo)));
+        const u32x2 b = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, hi)));
+        ColOperand o;
+        o.v = u32x4{a[0], a[1], b[0], b[1]};
+        return o;
+      };
+      const T* kt = reinterpret_cast<const T*>(smem + FC::K_OFF);
+      constexpr int NT1 = NMT - NT0;
+      for (int kb = 0; kb < nkb; ++kb, xt += FC::XTILE / 2, kt += TB / 2) {
+        // B operands: dS^T of 16 keys each (steps 0, 1) for this wave's 32 queries; A operands: K^T tiles of this part
+        const ColOperand b0 = x_operand(xt, 0), b1 = x_operand(xt, 1);
+        if (!part1) {
+          static_for<NT0>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * t, 0, lane), b0);
+            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * t, 1, lane), b1);
+          });
+          if constexpr (TAIL) {
+            const T* tp = kt + tail_lane_offset(lane, STR, 32 * NMT);
+            const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, tp)));
+            const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, tp + 8 * STR)));
+            ColOperand ka, d0, d1;
+            ka.v = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            tail_operands(b0, b1, d0, d1);
+            mma16(dQ16[0], ka, d0);
+            mma16(dQ16[1], ka, d1);
+          }
+        } else {
+          static_for<NT1>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * (NT0 + t), 0, lane), b0);
+            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * (NT0 + t), 1, lane), b1);
+          });
+        }
+      }
+    }
+    // The next half's first Q / dout tile was requested a whole tile ago: wait for it here, before the dQ rows are
+    // stored, so that the barrier below also publishes it and the next wait for memory comes a tile after the stores.
+    if (j_end < nqt) wait_tile(j_end);
+    lds_barrier();   // every wave has read its dS tiles: X becomes the staging area of this half's dQ rows
+    {
+      using C = Cfg<T, D>;
+      T* stage = reinterpret_cast<T*>(smem + FC::X_OFF);
+      T* srow = stage + ((wave & 3) * 32 + c32) * C::OSTRIDE;
+      constexpr int NT1 = NMT - NT0;
+      if (!part1) {
+#pragma unroll
+        for (int t = 0; t < NT0; ++t)
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj)
+            store4<T>(srow + t * 32 + jj * 8 + 4 * g, dQ[t][4 * jj] * p.scale, dQ[t][4 * jj + 1] * p.scale, dQ[t][4 * jj + 2] * p.scale,
+                      dQ[t][4 * jj + 3] * p.scale);
+        if constexpr (TAIL)
+          store_tail16<T, D, NMT>(stage + (wave & 3) * 32 * C::OSTRIDE, lane, [&](int hq, int e) { return dQ16[hq][e] * p.scale; });
+      } else {
+#pragma unroll
+        for (int t = 0; t < NT1; ++t)
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj)
+            store4<T>(srow + (NT0 + t) * 32 + jj * 8 + 4 * g, dQ[t][4 * jj] * p.scale, dQ[t][4 * jj + 1] * p.scale, dQ[t][4 * jj + 2] * p.scale,
+                      dQ[t][4 * jj + 3] * p.scale);
+      }
+      lds_barrier();
+      T* gdq = reinterpret_cast<T*>(p.dq) + base(5);
+      for (int v = tid; v < 128 * VPR; v += 512) {
+        const int row = v / VPR, cv = v % VPR, qrow = half * 128 + row;
+        if (qrow < p.Lq)
+          *reinterpret_cast<u32x4*>(gdq + (int64_t)qrow * p.st[5][1] + cv * C::VEC) =
+              *reinterpret_cast<const u32x4*>(stage + row * C::OSTRIDE + cv * C::VEC);
+      }
+      // (the next half's first barrier orders these staging reads before X is written again)
+    }
+  }
+
+  // ---- dK, dV of this wave's 32 keys
+  T* stage = reinterpret_cast<T*>(smem + FC::X_OFF);
+  store_rows_transposed<T, D, 8, NMT>(stage, reinterpret_cast<T*>(p.dk) + base(6), p.st[6][1], 0, p.Lkv, tid,
+                                      [&](int t, int i) { return dK[t][i] * p.scale; },
+                                      [&](void* ws) {
+                                        if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dK16[hq][e] * p.scale; });
+                                      });
+  store_rows_transposed<T, D, 8, NMT>(stage, reinterpret_cast<T*>(p.dv) + base(7), p.st[7][1], 0, p.Lkv, tid,
+                                      [&](int t, int i) { return dV[t][i]; },
+                                      [&](void* ws) {
+                                        if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dV16[hq][e]; });
+                                      });
+}
+
+template <int D>
+static int launch_bwd_fused_t(const BwdParams& p, int BH, hipStream_t stream) {
+  auto kern = attn_bwd_fused_bf16_kernel<D>;
+  static bool lds_ok[64] = {};
+  if (!ensure_dynamic_lds(kern, BwdFusedCfg<D>::LDS_BYTES, lds_ok)) return -7;
+  return launch_kernel(kern, dim3((uint32_t)BH), dim3(512), BwdFusedCfg<D>::LDS_BYTES, stream, p);
+}
+
 template <int D>
 static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
   using F = BwdFastCfg<D>;
@@ -375,6 +769,17 @@ int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream) 
   // 32-bit buffer addressing: every (batch, head) slab of rows must span < 2 GiB
   const int64_t max_row = std::max(std::max(std::max(p.st[0][1], p.st[1][1]), std::max(p.st[2][1], p.st[3][1])), p.st[4][1]);
   if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 256) >= (int64_t)1 << 31) return 1;
+  // whole (batch, head) units per work-group, every score tile formed once
+  const int Lmax = std::max(p.Lq, p.Lkv);
+  if (Lmax <= 256 && (DMF_BWD_FUSED == 2 || (DMF_BWD_FUSED == 1 && Lmax > 128))) {
+    switch (D) {
+      case 64: return launch_bwd_fused_t<64>(p, BH, stream);
+      case 72: return launch_bwd_fused_t<72>(p, BH, stream);
+      case 80: return launch_bwd_fused_t<80>(p, BH, stream);
+      case 96: return launch_bwd_fused_t<96>(p, BH, stream);
+      default: break;   // head dim 128: K, the tile stages and the exchange area exceed the LDS
+    }
+  }
   switch (D) {
     case 64: return launch_bwd_fast_t<64>(p, BH, stream);
     case 72: return launch_bwd_fast_t<72>(p, BH, stream);

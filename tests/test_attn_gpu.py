@@ -123,7 +123,8 @@ def test_reference_family(l, h, d):
 
 # ---- edge cases: ragged and tiny sequences, cross-attention lengths --------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("Lq,Lkv", [(1, 1), (16, 16), (64, 64), (100, 77), (129, 65), (257, 300), (128, 33)])
+@pytest.mark.parametrize("Lq,Lkv", [(1, 1), (16, 16), (64, 64), (100, 77), (129, 65), (257, 300), (128, 33),
+                                    (160, 200), (256, 130), (130, 256), (255, 40), (224, 256)])   # (the last five: single-pass backward)
 def test_ragged_lengths(Lq, Lkv, dtype):
     _parity(2, Lq, 2, 72, dtype, seed=Lq * 7 + Lkv, Lkv=Lkv)
 
