@@ -374,6 +374,21 @@ __device__ __forceinline__ void issue_tile_rows(__amdgpu_buffer_rsrc_t rsrc, uin
   }
 }
 
+// HBM -> LDS loads of ROWS whole rows by ONE wave: LDS placement is lane-linear (row pitch PITCH vectors, VPR of them
+// valid), lanes that fall on padding vectors are switched off; rows past the end of the resource read as zeros.
+template <int PITCH, int VPR, int ROWS>
+__device__ __forceinline__ void issue_rows(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_bytes, uint32_t soffset, char* lds_dst, int lane) {
+  constexpr int SLOTS = ROWS * PITCH;
+#pragma unroll
+  for (int i = 0; i < (SLOTS + 63) / 64; ++i) {
+    const int slot = 64 * i + lane;
+    const int r = slot / PITCH, cv = slot % PITCH;
+    if (slot < SLOTS && cv < VPR)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(lds_dst + 64 * i * 16), 16,
+                                               (uint32_t)r * row_bytes + cv * 16, soffset, 0, 0);
+  }
+}
+
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* base, uint32_t row_bytes, int nrows, int row_payload_bytes) {
   // raw buffer, byte-granular bounds: [base, base + (nrows-1)*row_bytes + payload)
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (nrows - 1) * row_bytes + row_payload_bytes, 0x00020000);

@@ -6,7 +6,13 @@
 //   * <= 256 VGPRs so two work-groups (8 waves) share a CU and one wave's
 //     softmax VALU work overlaps another wave's MFMAs;
 //   * K, V, dK, dV tiles of 32 keys go HBM -> LDS with global_load_lds_dwordx4
-//     (no staging registers), double-buffered, one barrier per tile;
+//     (no staging registers), double-buffered, one barrier per tile; the four
+//     load instructions of the next tile are issued one at a time between the
+//     score MFMAs of the current one (issued together right after the barrier
+//     they keep all eight waves off the matrix pipe for ~350 cycles per tile);
+//   * 256-row work-groups fetch their Q / dQ rows the same way (whole rows by
+//     DMA into LDS, operands read from there) instead of one scattered 16-byte
+//     load per lane and chunk;
 //   * Q and dQ are pre-multiplied by the softmax scale when loaded, so neither
 //     S nor dS needs a per-element scale;
 //   * lazy rescaling: the running maximum is only raised (and O, dO rescaled)
@@ -30,6 +36,7 @@ struct FastCfg {
   static constexpr int VP = NDT * 4 <= 4 ? 4 : (NDT * 4 <= 12 ? 12 : 20);  // V/dV pitch: 4 (mod 8) vectors => conflict-free transposed reads
   static constexpr int KSTR = KP * 8, VSTR = VP * 8;                       // pitches in elements
   static constexpr int BKV = 32;
+  static constexpr int QP = VPR | 1;                                       // Q/dQ staging row pitch in vectors (odd => conflict-free b128 reads)
   static constexpr int KBYTES = BKV * KP * 16, VBYTES = BKV * VP * 16;
   // Head dims with a remainder of at most 16 over a multiple of 32 (72, 80): the
   // remainder columns of O^T / dO^T are produced by 16x16x32 MFMAs instead of a
@@ -54,6 +61,9 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NDT = F::NDT, KP = F::KP, VP = F::VP;
   constexpr int KSTR = F::KSTR, VSTR = F::VSTR, BKV = F::BKV;
   constexpr int STAGE = (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES);
+  // Staging of this work-group's Q (and dQ) rows behind the two tile stages, when 160 KB of LDS have room for it.
+  constexpr int QP = F::QP, QS_OFF = 2 * STAGE + 512, QS_BYTES = 32 * NW * QP * 16;
+  constexpr bool QLDS = NW == 8 && QS_OFF + (JVP ? 2 : 1) * QS_BYTES <= 160 * 1024;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   auto Kt = [&](int s) { return smem + s * STAGE; };
@@ -82,16 +92,20 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   const __amdgpu_buffer_rsrc_t rs_v = make_rows_rsrc(gv, rb_v, p.Lkv, D * 2);
   const __amdgpu_buffer_rsrc_t rs_tk = make_rows_rsrc(JVP ? gtk : gk, JVP ? rb_tk : rb_k, p.Lkv, D * 2);
   const __amdgpu_buffer_rsrc_t rs_tv = make_rows_rsrc(JVP ? gtv : gv, JVP ? rb_tv : rb_v, p.Lkv, D * 2);
-  auto issue = [&](int it) {
+  // A tile is fetched in NPART parts (one DMA instruction per wave each): K, dK, V, dV.
+  constexpr int NPART = JVP ? 4 : 2;
+  static_assert(NCHUNK >= NPART, "one part of the next tile is issued after each of the first NPART score chunks");
+  constexpr int DMA_PER_TILE = (JVP ? 2 : 1) * ((32 / NW * KP + 63) / 64 + (32 / NW * VP + 63) / 64);   // vmcnt units per wave
+  auto issue_part = [&](int it, auto pc) {
+    constexpr int part = decltype(pc)::value;
     const int s = it & 1;
     const uint32_t r0 = (uint32_t)it * BKV;
-    issue_tile_rows<KP, VPR, NW>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
-    issue_tile_rows<VP, VPR, NW>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
-    if constexpr (JVP) {
-      issue_tile_rows<KP, VPR, NW>(rs_tk, rb_tk, r0 * rb_tk, dKt(s), wave, lane);
-      issue_tile_rows<VP, VPR, NW>(rs_tv, rb_tv, r0 * rb_tv, dVt(s), wave, lane);
-    }
+    if constexpr (part == 0) issue_tile_rows<KP, VPR, NW>(rs_k, rb_k, r0 * rb_k, Kt(s), wave, lane);
+    if constexpr (part == 1 && JVP) issue_tile_rows<KP, VPR, NW>(rs_tk, rb_tk, r0 * rb_tk, dKt(s), wave, lane);
+    if constexpr (part == (JVP ? 2 : 1)) issue_tile_rows<VP, VPR, NW>(rs_v, rb_v, r0 * rb_v, Vt(s), wave, lane);
+    if constexpr (part == 3 && JVP) issue_tile_rows<VP, VPR, NW>(rs_tv, rb_tv, r0 * rb_tv, dVt(s), wave, lane);
   };
+  auto issue = [&](int it) { static_for<NPART>([&](auto pc) { issue_part(it, pc); }); };
 
 
   // ---- padding of both stages: zeros, and the ones column of V
@@ -118,10 +132,45 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   {
     const int qrow = q0 + wave * 32 + c32;
     const uint32_t rb_q = (uint32_t)p.st[0][1] * 2;
-    load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(0), rb_q, p.Lq, D * 2), rb_q, qrow, g, Qr);
-    if constexpr (JVP) {
-      const uint32_t rb_tq = (uint32_t)p.st[3][1] * 2;
-      load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.tq) + base(3), rb_tq, p.Lq, D * 2), rb_tq, qrow, g, dQr);
+    if constexpr (QLDS) {
+      // Every wave fetches and reads only its own 32 rows: no barrier, just its own vmcnt.
+      char* qs = smem + QS_OFF + wave * 32 * QP * 16;
+      issue_rows<QP, VPR, 32>(make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(0), rb_q, p.Lq, D * 2), rb_q,
+                              (uint32_t)(q0 + wave * 32) * rb_q, qs, lane);
+      if constexpr (JVP) {
+        const uint32_t rb_tq = (uint32_t)p.st[3][1] * 2;
+        issue_rows<QP, VPR, 32>(make_rows_rsrc(reinterpret_cast<const T*>(p.tq) + base(3), rb_tq, p.Lq, D * 2), rb_tq,
+                                (uint32_t)(q0 + wave * 32) * rb_tq, qs + QS_BYTES, lane);
+      }
+      issue(0);   // the first key tile follows the Q rows; loads complete in order, so it may stay in flight below
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (DMA_PER_TILE & 15) | ((DMA_PER_TILE >> 4) << 14));
+      const uint32_t qa = lds_addr(qs) + c32 * QP * 16;
+      static_for<NCHUNK>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        // (the upper half of the last chunk of a head dim that is not a multiple of 16 does not exist: read the lower one, zeroed below)
+        const uint32_t a = 2 * c + 1 < VPR ? qa + g * 16 : qa;
+        Qr[c] = lds_read128_issue<32 * c>(a);
+        if constexpr (JVP) dQr[c] = lds_read128_issue<32 * c + QS_BYTES>(a);
+      });
+      if constexpr (JVP) lds_read128_wait<0>(Qr[NCHUNK - 1], dQr[NCHUNK - 1]);
+      else lds_read128_wait<0>(Qr[NCHUNK - 1]);
+#pragma unroll
+      for (int c = 0; c + 1 < NCHUNK; ++c) {   // the other chunks are valid after the same wait
+        if constexpr (JVP) asm volatile("" : "+v"(Qr[c]), "+v"(dQr[c]));
+        else asm volatile("" : "+v"(Qr[c]));
+      }
+      if constexpr (2 * NCHUNK > VPR) {
+        if (g == 1) {
+          Qr[NCHUNK - 1] = u32x4{0, 0, 0, 0};
+          if constexpr (JVP) dQr[NCHUNK - 1] = u32x4{0, 0, 0, 0};
+        }
+      }
+    } else {
+      load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.q) + base(0), rb_q, p.Lq, D * 2), rb_q, qrow, g, Qr);
+      if constexpr (JVP) {
+        const uint32_t rb_tq = (uint32_t)p.st[3][1] * 2;
+        load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.tq) + base(3), rb_tq, p.Lq, D * 2), rb_tq, qrow, g, dQr);
+      }
     }
     auto lo = [](uint32_t w) { return __uint_as_float(w << 16); };
     auto hi = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
@@ -180,7 +229,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   }
 
   // first key tile on its way (issued after the Q loads: measured faster than issuing it first)
-  issue(0);
+  if constexpr (!QLDS) issue(0);
 
   constexpr int NMT = F::NMT;
   constexpr bool TAIL = F::TAIL;
@@ -212,7 +261,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile `it` has landed in LDS
     lds_barrier();                         // ... and everyone else's; also: all waves are done with the other stage
-    if (it + 1 < ntiles) issue(it + 1);
+    const bool fetch = it + 1 < ntiles;    // tile it + 1 goes into the other stage, in parts between the score MFMAs
     const int s = it & 1;
 
     // ---- S^T (already scaled) and dS^T; the LDS reads of chunk c+1 are in
@@ -238,6 +287,9 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
         } else {
           lds_read128_wait<more ? 1 : 0>(kc[c & 1]);
           mma_chunk<T>(S, kc[c & 1], Qr[c]);
+        }
+        if constexpr (c < NPART) {
+          if (fetch) issue_part(it + 1, cc);
         }
       });
     }
@@ -400,7 +452,9 @@ static int launch_fast_q(const FwdParams& p, int BH, hipStream_t stream) {
   using F = FastCfg<D>;
   constexpr int tiles = 2 * (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES) + 512;
   constexpr int stage = 32 * NW * Cfg<__bf16, D>::OROWV * 16;
-  constexpr int smem = tiles > stage ? tiles : stage;
+  constexpr int qst = (JVP ? 2 : 1) * 32 * NW * F::QP * 16;                       // Q / dQ staging of the 8-wave kernel (see QLDS there)
+  constexpr int need = (NW == 8 && tiles + qst <= 160 * 1024) ? tiles + qst : tiles;
+  constexpr int smem = need > stage ? need : stage;
   auto kern = attn_fwd_bf16_kernel<D, JVP, NW, QN>;
   static bool lds_ok[64] = {};
   if (!ensure_dynamic_lds(kern, smem, lds_ok)) return -7;
