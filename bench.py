@@ -32,9 +32,12 @@ if ROOT not in sys.path:
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the fused fwd+JVP kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (each scaled by what the counter reads for a plain 1 GiB copy; summaries in profiles/attn_fwd_jvp_bf16_d72_*.txt)
-MEASURED_TRAFFIC_BYTES = {"xl2_512px": 1.2131e9, "xl2_256px": 1.2126e9}
+# HBM bytes per step of each entry point, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over
+# `bench.py --workload W --kernel K` (each scaled by what the counter reads for a plain 1 GiB copy in the same run;
+# summaries in profiles/attn_<kernel>_bf16_d72_<workload>.txt).  The two-kernel backward at N=1024 reads q, k, v, dout twice.
+MEASURED_TRAFFIC_BYTES = {("fwd_jvp", "xl2_512px"): 1.2124e9, ("fwd_jvp", "xl2_256px"): 1.2123e9,
+                          ("fwd", "xl2_512px"): 6.0845e8, ("fwd", "xl2_256px"): 6.0906e8,
+                          ("bwd", "xl2_512px"): 1.8728e9, ("bwd", "xl2_256px"): 1.2170e9}
 
 DEVICE_WAKE_SECONDS = 0.3        # untimed launches of the measured kernel before the --warmup steps (clock ramp from idle)
 
@@ -153,12 +156,28 @@ def cpu_baseline_config1():
     return out
 
 
-def roofline(name, ms):
-    """Roofline entry for the fused fwd+JVP kernel: the MFMA roof when the workload's arithmetic intensity is above
-    the machine balance (2.5 PFLOP/s / 8 TB/s = 312 FLOP/B), the HBM roof otherwise (N=256: 191 FLOP/B)."""
+# Kernels behind each entry point at the two workloads (rocprofv3 names), and where the offline counter figures live.
+KERNELS = {"fwd_jvp": "dmf::attn_fwd_bf16_kernel<72, true, 8, false>", "fwd": "dmf::attn_fwd_bf16_kernel<72, false, 8, false>",
+           "bwd": {"xl2_512px": "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72>",
+                   "xl2_256px": "dmf::attn_bwd_fused_bf16_kernel<72>"}}
+PROFILE_FILES = {("fwd_jvp", "xl2_512px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_512px.txt", ("fwd_jvp", "xl2_256px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_256px.txt",
+                 ("fwd", "xl2_512px"): "profiles/attn_fwd_bf16_d72_xl2_512px.txt", ("fwd", "xl2_256px"): "profiles/attn_fwd_bf16_d72_xl2_256px.txt",
+                 ("bwd", "xl2_512px"): "profiles/attn_bwd_bf16_d72_xl2_512px.txt", ("bwd", "xl2_256px"): "profiles/attn_bwd_bf16_d72_xl2_256px.txt"}
+# Share of the clocked cycles in which the MFMA pipe was busy (SQ_VALU_MFMA_BUSY_CYCLES / (4 SQ_BUSY_CU_CYCLES)), from the
+# rocprofv3 --pmc runs summarised in the files above (offline, like `traffic`); None where no such run is committed.
+MEASURED_MFMA_BUSY = {("fwd_jvp", "xl2_512px"): 0.588, ("fwd_jvp", "xl2_256px"): 0.363, ("fwd", "xl2_512px"): 0.492,
+                      ("fwd", "xl2_256px"): 0.294, ("bwd", "xl2_512px"): 0.436, ("bwd", "xl2_256px"): 0.189}
+
+
+def roofline(name, ms, kind="fwd_jvp"):
+    """Roofline entry for one kernel-level measurement: the MFMA roof when the workload's arithmetic intensity is above
+    the machine balance (2.5 PFLOP/s / 8 TB/s = 312 FLOP/B), the HBM roof otherwise (fwd+JVP at N=256: 191 FLOP/B)."""
     B, H, N, D, _ = WORKLOADS[name]
-    flops, nbytes = attn_flops(B, H, N, D, "fwd_jvp"), attn_bytes(B, H, N, D, "fwd_jvp")
-    common = {"traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8, false>"}
+    flops, nbytes = attn_flops(B, H, N, D, kind), attn_bytes(B, H, N, D, kind)
+    kern = KERNELS[kind]
+    common = {"traffic": MEASURED_TRAFFIC_BYTES.get((kind, name)),
+              "traffic_source": PROFILE_FILES[(kind, name)] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, offline)",
+              "mfma_busy": MEASURED_MFMA_BUSY.get((kind, name)), "kernel": kern if isinstance(kern, str) else kern[name]}
     if flops / nbytes >= MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
         a = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": a / MFMA_BF16_PEAK_TFLOPS,
@@ -203,6 +222,31 @@ class _Telemetry:
         self.sclk_file = os.path.join(dev, "pp_dpm_sclk") if dev and os.path.exists(os.path.join(dev, "pp_dpm_sclk")) else None
         cap = pw[0].replace("power1_input", "power1_cap") if pw else None
         self.cap_w = int(open(cap).read()) / 1e6 if cap and os.path.exists(cap) else None
+        # The SMU's throttler residency counters (amdsmi): one tick per controller iteration (about 1 kHz) in which
+        # the package-power (PPT), socket / VR / HBM thermal or PROCHOT controller was holding the clocks down.
+        self.smi = None
+        try:
+            import amdsmi
+            amdsmi.amdsmi_init()
+            self.smi = (amdsmi, amdsmi.amdsmi_get_processor_handles()[0])
+            self._violations()
+        except Exception:   # not installed, no permission, or a driver that does not export the counters
+            self.smi = None
+
+    def _violations(self):
+        amdsmi, h = self.smi
+        v = amdsmi.amdsmi_get_violation_status(h)
+        keys = ("acc_counter", "acc_ppt_pwr", "acc_socket_thrm", "acc_vr_thrm", "acc_hbm_thrm", "acc_prochot_thrm")
+        return {k: v[k] for k in keys if isinstance(v.get(k), int)}
+
+    def _metrics(self):
+        amdsmi, h = self.smi
+        m = amdsmi.amdsmi_get_gpu_metrics_info(h)
+        out = {k: m[k] for k in ("temperature_hotspot", "temperature_mem", "current_socket_power") if isinstance(m.get(k), (int, float))}
+        clk = [c for c in m.get("current_gfxclks", []) if isinstance(c, (int, float))]
+        if clk:
+            out["gfxclk_mhz_per_xcd"] = clk
+        return out
 
     def available(self):
         return self.power_file is not None
@@ -216,7 +260,7 @@ class _Telemetry:
                     f = float(line.split(":")[1].strip().rstrip("*").strip().lower().replace("mhz", ""))
         return p, f
 
-    def measure(self, fn, seconds=1.0, burst=20):
+    def measure(self, fn, seconds=2.0, burst=20):
         """Run ``fn`` (which enqueues GPU work) repeatedly for about ``seconds`` and return mean / max power in watts
         and the mean shader clock in MHz over the samples taken after the first quarter of the interval."""
         import threading
@@ -234,10 +278,18 @@ class _Telemetry:
         th = threading.Thread(target=sampler, daemon=True)
         t0 = time.perf_counter()
         th.start()
+        v0 = v1 = smu = None
         while time.perf_counter() - t0 < seconds:
             for _ in range(burst):
                 fn()
             torch.cuda.synchronize()
+            if self.smi is not None and v0 is None and time.perf_counter() - t0 > 0.3 * seconds:
+                v0 = self._violations()     # both readings are taken while the load runs: the counters lag by a fraction of a second
+        if self.smi is not None and v0 is not None:
+            try:
+                v1, smu = self._violations(), self._metrics()
+            except Exception:
+                v1 = None
         stop.set()
         th.join()
         t1 = time.perf_counter()
@@ -245,12 +297,18 @@ class _Telemetry:
         if not keep:
             return None
         clocks = [x[2] for x in keep if x[2] is not None]
-        return {"power_w_mean": sum(x[1] for x in keep) / len(keep), "power_w_max": max(x[1] for x in keep),
-                "sclk_mhz_mean": sum(clocks) / len(clocks) if clocks else None, "samples": len(keep)}
+        out = {"power_w_mean": sum(x[1] for x in keep) / len(keep), "power_w_max": max(x[1] for x in keep),
+               "sclk_mhz_mean": sum(clocks) / len(clocks) if clocks else None, "samples": len(keep)}
+        if v1 is not None and v1.get("acc_counter", 0) > v0.get("acc_counter", 0):
+            ticks = v1["acc_counter"] - v0["acc_counter"]
+            out["throttler_residency_pct"] = {k[4:]: 100.0 * (v1[k] - v0[k]) / ticks for k in v1 if k != "acc_counter" and k in v0}
+            out["smu"] = smu
+        return out
 
 
 def power_probes(fns):
-    """Board power and shader clock while each of the named GPU workloads runs for a second (None without sysfs access)."""
+    """Board power, shader clock and the SMU's throttler residencies while each of the named GPU workloads runs for two
+    seconds (None without sysfs access)."""
     tel = _Telemetry()
     if not tel.available():
         return None
@@ -324,11 +382,19 @@ def block_kernel_rows(device, steps=50, warmup=10):
 
 
 def main():
+    from dmf_amd.layers import ATTN_FUNCS
+
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="xl2_512px", choices=list(WORKLOADS))
+    ap.add_argument("--kernel", default="fwd_jvp", choices=["fwd_jvp", "fwd", "bwd"],
+                    help="the entry point one step launches (default: the fused forward+JVP, the headline); "
+                         "'fwd' = primal-only forward, 'bwd' = backward on the primal output -- for per-kernel profiles")
+    ap.add_argument("--attn-func", default="hip", choices=ATTN_FUNCS,
+                    help="attention operator of the model built by --dmft-graph (the reference's --attn-func switch, "
+                         "train_dmf.py:427, with the new value 'hip')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--copy-calib", action="store_true",
@@ -351,14 +417,17 @@ def main():
     dev, dtype = "cuda:0", torch.bfloat16
     if args.dmft_graph:
         from dmf_amd import harness
-        rows = harness.bench_dmft(steps=max(1, args.steps // 4), only=args.dmft_graph, variants=("hip_fused_graph",))
+        # 'hip': the fused model replayed as a HIP graph; 'base' / 'torch_sdpa': the reference's expressions around that operator, eager
+        variant = "hip_fused_graph" if args.attn_func == "hip" else args.attn_func
+        rows = harness.bench_dmft(steps=max(1, args.steps // 4), only=args.dmft_graph, variants=(variant,))
         if args.dmft_graph not in rows:
             sys.exit(f"bench.py: unknown --dmft-graph case {args.dmft_graph!r}")
         row = rows[args.dmft_graph]
-        print(json.dumps({"metric": "dmft_images_per_s", "value": row["hip_fused_graph_images_per_s"], "unit": "images/s",
-                          "n_gpus": 1, "steps": args.steps, "ms_per_step": row["hip_fused_graph_ms_per_step"],
+        how = "hip attention + fused block glue, HIP-graph replay" if args.attn_func == "hip" else f"{args.attn_func} attention, eager"
+        print(json.dumps({"metric": "dmft_images_per_s", "value": row[f"{variant}_images_per_s"], "unit": "images/s",
+                          "n_gpus": 1, "steps": args.steps, "ms_per_step": row[f"{variant}_ms_per_step"],
                           "config": {"workload": f"{args.dmft_graph}: {row['tokens']} tokens, {row['mode']}, batch {row['batch']}, "
-                                                 f"{row['dtype']}, hip attention + fused block glue, HIP-graph replay"}}))
+                                                 f"{row['dtype']}, {how}", "attn_func": args.attn_func}}))
         return
     name = args.workload
     B, H, N, D, _ = WORKLOADS[name]
@@ -374,26 +443,35 @@ def main():
 
     # an idle device sits at its lowest clock level (157 MHz shader clock) and takes tens of milliseconds of load to leave
     # it: bring it up with untimed launches first, so that a short --warmup measures the same steady state as a long one
+    kind = args.kernel
+    if kind == "fwd_jvp":
+        step = lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)
+    elif kind == "fwd":
+        step = lambda: _lib.fwd(q, k, v, scale)
+    else:
+        o0, lse0 = _lib.fwd(q, k, v, scale)[:2]
+        step = lambda: _lib.bwd(do, q, k, v, o0, lse0, scale)
+    label = {"fwd_jvp": "fwd+JVP", "fwd": "primal forward", "bwd": "backward (dQ, dK, dV)"}[kind]
     wake_until = time.perf_counter() + DEVICE_WAKE_SECONDS
     while time.perf_counter() < wake_until:
         for _ in range(10):
-            _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)
+            step()
         torch.cuda.synchronize()
-    ms, wall_ms = time_gpu(lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale), args.steps, args.warmup)
-    flops = attn_flops(B, H, N, D, "fwd_jvp")
+    ms, wall_ms = time_gpu(step, args.steps, args.warmup)
+    flops = attn_flops(B, H, N, D, kind)
     tflops = flops / (ms * 1e-3) / 1e12
-    ms_median, ms_min = per_launch_stats(lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale))
-    progress(f"{name} attention fwd+JVP: {ms:.4f} ms/step, {tflops:.1f} TFLOP/s")
+    ms_median, ms_min = per_launch_stats(step)
+    progress(f"{name} attention {label}: {ms:.4f} ms/step, {tflops:.1f} TFLOP/s")
     result = {
-        "metric": "attn_fwd_jvp_tflops", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
+        "metric": f"attn_{kind}_tflops", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{name}: attention fwd+JVP B={B} H={H} N={N} D={D} bf16"
+        "config": {"workload": f"{name}: attention {label} B={B} H={H} N={N} D={D} bf16"
                                + (" q,k RMS-normalised" if WORKLOADS[name][4] else ""),
-                   "flops_per_step": flops, "hbm_bytes_per_step": attn_bytes(B, H, N, D, "fwd_jvp"),
+                   "flops_per_step": flops, "hbm_bytes_per_step": attn_bytes(B, H, N, D, kind),
                    "wall_ms_per_step": wall_ms, "single_launch_ms_median": ms_median, "single_launch_ms_min": ms_min,
                    "untimed_device_wake_seconds": DEVICE_WAKE_SECONDS},
-        "roofline": roofline(name, ms),
+        "roofline": roofline(name, ms, kind),
     }
 
     if not args.no_extra:
@@ -414,18 +492,26 @@ def main():
                 t_ms, _ = time_gpu(fn, max(10, args.steps // 2), max(5, args.warmup // 2))
                 fl, by = attn_flops(Bw, Hw, Nw, Dw, kind), attn_bytes(Bw, Hw, Nw, Dw, kind)
                 row[kind] = {"ms": t_ms, "tflops": fl / t_ms / 1e9, "pct_bf16_mfma_peak": 100 * fl / t_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
-                             "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS}
+                             "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS,
+                             "roofline": roofline(wname, t_ms, kind)}
             extra[wname] = row
             progress(f"{wname}: fwd_jvp / fwd / bwd = " + " / ".join(f"{row[kd]['ms']:.4f}" for kd in ("fwd_jvp", "fwd", "bwd")) + " ms")
             del ins
         extra["device_probes"] = device_probes()
         zq = torch.zeros_like(q)
+        other = "xl2_256px" if name == "xl2_512px" else "xl2_512px"
+        q2, k2, v2, tq2, tk2, tv2, do2 = make_inputs(other, dev, dtype, seed=3)
+        o2, _, lse2 = _lib.fwd_jvp(q2, k2, v2, tq2, tk2, tv2, scale)
+        zq2 = torch.zeros_like(q2)
         extra["power"] = power_probes([
-            ("attn_fwd_jvp_xl2_512px", lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)),
-            ("attn_fwd_jvp_xl2_512px_all_zero_inputs", lambda: _lib.fwd_jvp(zq, zq, zq, zq, zq, zq, scale)),
-            ("attn_bwd_xl2_512px", lambda: _lib.bwd(do, q, k, v, o, lse, scale)),
+            (f"attn_fwd_jvp_{name}", lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)),
+            (f"attn_fwd_jvp_{name}_all_zero_inputs", lambda: _lib.fwd_jvp(zq, zq, zq, zq, zq, zq, scale)),
+            (f"attn_bwd_{name}", lambda: _lib.bwd(do, q, k, v, o, lse, scale)),
+            (f"attn_fwd_jvp_{other}", lambda: _lib.fwd_jvp(q2, k2, v2, tq2, tk2, tv2, scale)),
+            (f"attn_fwd_jvp_{other}_all_zero_inputs", lambda: _lib.fwd_jvp(zq2, zq2, zq2, zq2, zq2, zq2, scale)),
+            (f"attn_bwd_{other}", lambda: _lib.bwd(do2, q2, k2, v2, o2, lse2, scale)),
         ])
-        del zq
+        del zq, zq2, q2, k2, v2, tq2, tk2, tv2, do2, o2, lse2
         progress("device probes done" + ("" if extra["power"] is None else f"; power {json.dumps(extra['power'])}"))
         extra["block_kernels"] = block_kernel_rows(dev)
         progress("block kernels done")

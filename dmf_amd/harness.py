@@ -295,6 +295,8 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
                     ("hip", "hip", "torch", False)]
     if compare_base:
         all_variants.append(("base", "base", "torch", False))
+    if variants is not None and "torch_sdpa" in variants:   # the reference's third operator value, only on request
+        all_variants.append(("torch_sdpa", "torch_sdpa", "torch", False))
     variants = [v for v in all_variants if variants is None or v[0] in variants]
     modes = {"jvp": "fwd+jvp", "train": "fwd+jvp+bwd", "nograd": "primal-only forward, no grad (guidance / sampler call)",
              "dmf_loss": "fwd(grad) + 2x guidance fwd (no grad, 2B) + fwd+jvp, then bwd", "fm": "fwd+bwd (no jvp)",
