@@ -36,6 +36,7 @@ SIGNATURES = {
     "dmf_attn_fwd_jvp": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_fwd": (c_int, [_P] * 5 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_fwd_qnorm": (c_int, [_P] * 7 + [_F] + [_P] * 4 + [_S] + [_I] * 5 + [_F, _I, _P]),
+    "dmf_attn_fwd_qknorm": (c_int, [_P] * 8 + [_F] + [_P] * 6 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_bwd": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_block_workspace_floats": (c_int64, [_I] * 4),
     "dmf_ln_modulate_fwd": (c_int, [_P] * 8 + [_S] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
@@ -308,6 +309,49 @@ def fwd_qnorm(q, k, v, tq, tk, tv, q_gain, eps: float, scale: float, need_lse: b
         return None
     _check(rc, "dmf_attn_fwd_qnorm")
     return o, to, lse
+
+
+def fwd_qknorm(q, k, v, tq, tk, tv, q_gain, k_gain, eps: float, scale: float, need_lse: bool = True, save_normed: bool = False):
+    """Forward (+ JVP when ``tq`` is given) on the raw q and k projections: the per-head RMS norms of q and of k (gains
+    ``q_gain``, ``k_gain``, (D); ``k_gain`` None: k is already normalised) are applied inside the attention kernel.  Returns (o, to, lse, q_hat, k_hat) -- ``to``
+    None without tangents, ``q_hat`` / ``k_hat`` the normalised primal rows when ``save_normed`` (a backward pass
+    follows), else None -- or None when no kernel implements the variant for this shape / dtype."""
+    jvp = tq is not None
+    if jvp:
+        _check_inputs(q, k, v, tq, tk, tv)
+        q, k, v, tq, tk, tv = map(_prep, (q, k, v, tq, tk, tv))
+    else:
+        _check_inputs(q, k, v)
+        q, k, v = map(_prep, (q, k, v))
+    gains = []
+    for name, gn in (("q_gain", q_gain), ("k_gain", k_gain)):
+        if gn is None and name == "k_gain":   # k is already normalised
+            gains.append(None)
+            continue
+        gn = _raw(gn)
+        if gn.dim() != 1 or gn.shape[0] != q.shape[-1] or gn.device != q.device:
+            raise ValueError(f"fwd_qknorm: {name} must be a (D) tensor on the device of q")
+        gains.append(_raw(gn.float().contiguous()))   # exact for a bf16 gain (a model cast to bf16 as a whole)
+    if q.dtype != torch.bfloat16 or any(gn is not None and gn.data_ptr() % 16 for gn in gains):
+        return None
+    B, Lq, H, D = q.shape
+    Lkv = k.shape[1]
+    o = _empty((B, Lq, H, D), q.dtype, q.device)
+    to = _empty((B, Lq, H, D), q.dtype, q.device) if jvp else None
+    lse = _empty((B, H, Lq), torch.float32, q.device) if (need_lse or jvp) else None
+    qh = _empty((B, Lq, H, D), q.dtype, q.device) if save_normed else None
+    kh = _empty((B, Lkv, H, D), q.dtype, q.device) if save_normed and gains[1] is not None else None
+    z = q   # stands in for absent tangents in the stride table (ignored by the library)
+    with _on(q.device):
+        rc = load().dmf_attn_fwd_qknorm(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _ptr(tq), _ptr(tk), _ptr(tv), gains[0].data_ptr(), _ptr(gains[1]), float(eps),
+            o.data_ptr(), _ptr(to), _ptr(lse), None, _ptr(qh), _ptr(kh),
+            _strides(q, k, v, tq if jvp else z, tk if jvp else z, tv if jvp else z, o, to if jvp else o),
+            B, H, Lq, Lkv, D, float(scale), _dtype_code(q), _stream(q))
+    if rc == ENOKERNEL:
+        return None
+    _check(rc, "dmf_attn_fwd_qknorm")
+    return o, to, lse, qh, kh
 
 
 def bwd(dout, q, k, v, o, lse, scale: float, out=None):

@@ -54,6 +54,20 @@ __device__ __forceinline__ float xhalf_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// v + (v rotated right by N lanes within each row of 16 lanes), as one DPP-modified add
+template <int N>
+__device__ __forceinline__ float row_ror_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, false));
+}
+
+// sum over the 16 lanes of an aligned lane group; every lane of the group gets the same bits
+__device__ __forceinline__ float group16_sum(float v) {
+  v = row_ror_add<8>(v);
+  v = row_ror_add<4>(v);
+  v = row_ror_add<2>(v);
+  return row_ror_add<1>(v);
+}
+
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   f32x2 x = {a, b};
   bf16x2 y = __builtin_convertvector(x, bf16x2);  // v_cvt_pk_bf16_f32, round-to-nearest-even

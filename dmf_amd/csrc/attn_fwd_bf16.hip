@@ -53,8 +53,10 @@ struct FastCfg {
 // NW = waves per work-group: 4 (128 query rows, two work-groups per CU) or
 // 8 (256 query rows, one work-group per CU: half the tile traffic per FLOP).
 // QN: per-head RMS norm of q (and its tangent) applied while the Q operands are formed.
-template <int D, bool JVP, int NW, bool QN = false>
+// KN: per-head RMS norm of k (and its tangent) applied to every key tile in LDS, between its arrival and its use.
+template <int D, bool JVP, int NW, bool QN = false, bool KN = false>
 __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const FwdParams p) {
+  static_assert(!KN || QN, "the key norm is only built together with the query norm");
   constexpr int NTHR = 64 * NW, BQ = 32 * NW;
   using F = FastCfg<D>;
   using T = __bf16;
@@ -214,6 +216,12 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
           Qr[c][e] = qn;
         }
       }
+      if (p.q_hat != nullptr && qrow < p.Lq) {   // normalised rows for the backward pass (before the softmax scale goes in)
+        T* dst = reinterpret_cast<T*>(p.q_hat) + (((int64_t)b * p.Lq + qrow) * p.H + h) * D + 8 * g;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c)
+          if (2 * c + g < VPR) *reinterpret_cast<u32x4*>(dst + 16 * c) = Qr[c];
+      }
     }
     auto scaled = [&](u32x4 x) {
       u32x4 y;
@@ -257,12 +265,66 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   // probabilities that row receives from swap16 -- at head-dim columns 32*NMT .. 32*NMT+15.
   const uint32_t t_lane_addr = lds_addr(smem) + F::KBYTES + tail_lane_offset(lane, VSTR, 32 * F::NMT) * 2;
 
+  // KN: a 16-lane group owns one key row of the tile (lane i of the group: elements 8i .. 8i+7), a wave 4 rows per pass.
+  float kgain[8];
+  if constexpr (KN) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) kgain[e] = (lane & 15) < VPR ? p.k_gain[8 * (lane & 15) + e] : 0.f;
+  }
+
   const int ntiles = (p.Lkv + BKV - 1) / BKV;
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile `it` has landed in LDS
     lds_barrier();                         // ... and everyone else's; also: all waves are done with the other stage
     const bool fetch = it + 1 < ntiles;    // tile it + 1 goes into the other stage, in parts between the score MFMAs
     const int s = it & 1;
+    if constexpr (KN) {
+      // k_hat = k r g, dk_hat = (dk r + k dr) g with r = (mean k^2 + eps)^-1/2, dr = -r^3 mean(k dk): models/layers.py:39-42 and
+      // its tangent, element for element the arithmetic of the stand-alone norm kernel; rounded to bf16 in place.
+      constexpr int RPW = 32 / NW;
+      auto lo = [](uint32_t w) { return __uint_as_float(w << 16); };
+      auto hi = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
+#pragma unroll
+      for (int ps = 0; ps < RPW / 4; ++ps) {
+        const int row = RPW * wave + 4 * ps + (lane >> 4), cv = lane & 15;
+        const bool live = cv < VPR;
+        char* ka = Kt(s) + (row * KP + (live ? cv : 0)) * 16;
+        u32x4 kv = *reinterpret_cast<const u32x4*>(ka), tkv = u32x4{0, 0, 0, 0};
+        if constexpr (JVP) tkv = *reinterpret_cast<const u32x4*>(ka + DV_OFF);
+        if (!live) kv = tkv = u32x4{0, 0, 0, 0};
+        float x[8], t[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          x[2 * e] = lo(kv[e]);
+          x[2 * e + 1] = hi(kv[e]);
+          t[2 * e] = lo(tkv[e]);
+          t[2 * e + 1] = hi(tkv[e]);
+        }
+        float ss = 0.f, st = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          ss = fmaf(x[e], x[e], ss);
+          if constexpr (JVP) st = fmaf(x[e], t[e], st);
+        }
+        const float r = 1.f / sqrtf(group16_sum(ss) * (1.f / D) + p.q_eps);
+        const float dr = JVP ? -r * r * r * group16_sum(st) * (1.f / D) : 0.f;
+        if (live) {
+          u32x4 kn, tkn;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            kn[e] = pack_bf16x2(x[2 * e] * r * kgain[2 * e], x[2 * e + 1] * r * kgain[2 * e + 1]);
+            if constexpr (JVP)
+              tkn[e] = pack_bf16x2(fmaf(t[2 * e], r, x[2 * e] * dr) * kgain[2 * e], fmaf(t[2 * e + 1], r, x[2 * e + 1] * dr) * kgain[2 * e + 1]);
+          }
+          *reinterpret_cast<u32x4*>(ka) = kn;
+          if constexpr (JVP) *reinterpret_cast<u32x4*>(ka + DV_OFF) = tkn;
+          const int key = it * BKV + row;
+          if (p.k_hat != nullptr && qb == 0 && key < p.Lkv)   // the first query block of the head hands the rows to the backward pass
+            *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(p.k_hat) + (((int64_t)b * p.Lkv + key) * p.H + h) * D + 8 * cv) = kn;
+        }
+      }
+      lds_barrier();
+    }
 
     // ---- S^T (already scaled) and dS^T; the LDS reads of chunk c+1 are in
     //      flight while the MFMAs of chunk c run
@@ -447,7 +509,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
                                          [&](int t, int i) { return fmaf(-mu_n, O[t][i] * inv_l, dO[t][i] * inv_l); }, tail_to);
 }
 
-template <int D, bool JVP, int NW, bool QN>
+template <int D, bool JVP, int NW, bool QN, bool KN>
 static int launch_fast_q(const FwdParams& p, int BH, hipStream_t stream) {
   using F = FastCfg<D>;
   constexpr int tiles = 2 * (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES) + 512;
@@ -455,7 +517,7 @@ static int launch_fast_q(const FwdParams& p, int BH, hipStream_t stream) {
   constexpr int qst = (JVP ? 2 : 1) * 32 * NW * F::QP * 16;                       // Q / dQ staging of the 8-wave kernel (see QLDS there)
   constexpr int need = (NW == 8 && tiles + qst <= 160 * 1024) ? tiles + qst : tiles;
   constexpr int smem = need > stage ? need : stage;
-  auto kern = attn_fwd_bf16_kernel<D, JVP, NW, QN>;
+  auto kern = attn_fwd_bf16_kernel<D, JVP, NW, QN, KN>;
   static bool lds_ok[64] = {};
   if (!ensure_dynamic_lds(kern, smem, lds_ok)) return -7;
   const uint32_t nqb = (p.Lq + 32 * NW - 1) / (32 * NW);
@@ -466,9 +528,10 @@ template <int D, bool JVP, int NW>
 static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
   if (p.q_gain != nullptr) {
     if (reinterpret_cast<uintptr_t>(p.q_gain) % 16) return -6;
-    return launch_fast_q<D, JVP, NW, true>(p, BH, stream);
+    if (p.k_gain != nullptr) return launch_fast_q<D, JVP, NW, true, true>(p, BH, stream);
+    return launch_fast_q<D, JVP, NW, true, false>(p, BH, stream);
   }
-  return launch_fast_q<D, JVP, NW, false>(p, BH, stream);
+  return launch_fast_q<D, JVP, NW, false, false>(p, BH, stream);
 }
 
 // Work-group width policy: 256-row work-groups (one per CU, half the tile traffic per FLOP) when the sequence fills them.

@@ -20,6 +20,11 @@ struct FwdParams {
   // nullptr.  Only the tuned bf16 kernels implement it; the dispatcher reports kNoQNormKernel otherwise.
   const float* q_gain;
   float q_eps;
+  // Optional per-head RMS norm of k (and of its tangent) applied to every key tile once it has landed in LDS: gain (D)
+  // fp32 or nullptr (needs q_gain; same eps).  q_hat / k_hat: optional contiguous (B, L, H, D) outputs that receive the
+  // normalised primal rows (what a backward pass needs), or nullptr.
+  const float* k_gain;
+  void *q_hat, *k_hat;
 };
 
 constexpr int kNoQNormKernel = -8;

@@ -71,20 +71,6 @@ __device__ __forceinline__ float sum8(const float (&v)[8]) {
   return ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
 }
 
-// v + (v rotated right by N lanes within each row of 16 lanes), as one DPP-modified add
-template <int N>
-__device__ __forceinline__ float row_ror_add(float v) {
-  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, false));
-}
-
-// sum over the 16 lanes of an aligned lane group; every lane of the group gets the same bits
-__device__ __forceinline__ float group16_sum(float v) {
-  v = row_ror_add<8>(v);
-  v = row_ror_add<4>(v);
-  v = row_ror_add<2>(v);
-  return row_ror_add<1>(v);
-}
-
 // sum over the wave; every lane gets the same bits (no LDS traffic: DPP rotations inside the rows of 16 lanes, then the
 // 16- and 32-lane swaps)
 __device__ __forceinline__ float wave_sum(float v) {

@@ -58,7 +58,8 @@ static_assert(dmf::kNoQNormKernel == DMF_ATTN_ENOKERNEL, "dispatcher code and AB
 static int fwd_impl(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,
                     void* o, void* to, float* lse, float* dlse, const int64_t* strides, bool jvp,
                     int B, int H, int Lq, int Lkv, int D, float scale, int dtype, void* stream,
-                    const float* q_gain = nullptr, float q_eps = 0.f) {
+                    const float* q_gain = nullptr, float q_eps = 0.f, const float* k_gain = nullptr, void* q_hat = nullptr,
+                    void* k_hat = nullptr) {
   if (int rc = check_common(B, H, Lq, Lkv, D, dtype)) return rc;
   if (strides == nullptr) return DMF_ATTN_ENULL;
   const int eb = dtype == DMF_ATTN_BF16 ? 2 : 4;
@@ -80,6 +81,7 @@ static int fwd_impl(const void* q, const void* k, const void* v, const void* tq,
   p.H = H; p.Lq = Lq; p.Lkv = Lkv;
   p.scale = scale; p.scale_log2 = scale * 1.4426950408889634f;
   p.q_gain = q_gain; p.q_eps = q_eps;
+  p.k_gain = k_gain; p.q_hat = q_hat; p.k_hat = k_hat;
   return dmf::launch_fwd(p, B * H, D, dtype == DMF_ATTN_BF16, jvp, static_cast<hipStream_t>(stream));
 }
 
@@ -93,6 +95,21 @@ int dmf_attn_fwd_qnorm(const void* q, const void* k, const void* v, const void* 
   if (!jvp) tq = tk = tv = nullptr, dlse = nullptr;
   return fwd_impl(q, k, v, tq, tk, tv, o, to, lse, dlse, strides, jvp, B, H, Lq, Lkv, D, scale, dtype, stream, q_gain,
                   q_eps);
+}
+
+int dmf_attn_fwd_qknorm(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,
+                        const float* q_gain, const float* k_gain, float eps, void* o, void* to, float* lse, float* dlse,
+                        void* q_hat, void* k_hat, const int64_t* strides, int B, int H, int Lq, int Lkv, int D, float scale,
+                        int dtype, void* stream) {
+  if (q_gain == nullptr) return DMF_ATTN_ENULL;
+  if (k_gain == nullptr) k_hat = nullptr;   // k is taken as given
+  if (reinterpret_cast<uintptr_t>(q_gain) % 16 || reinterpret_cast<uintptr_t>(k_gain) % 16 ||
+      reinterpret_cast<uintptr_t>(q_hat) % 16 || reinterpret_cast<uintptr_t>(k_hat) % 16)
+    return DMF_ATTN_EALIGN;
+  const bool jvp = to != nullptr;
+  if (!jvp) tq = tk = tv = nullptr, dlse = nullptr;
+  return fwd_impl(q, k, v, tq, tk, tv, o, to, lse, dlse, strides, jvp, B, H, Lq, Lkv, D, scale, dtype, stream, q_gain, eps,
+                  k_gain, q_hat, k_hat);
 }
 
 int dmf_attn_fwd_jvp(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,

@@ -250,21 +250,28 @@ def flash_attn_qkvpacked_func(qkv, softmax_scale=None):
     return out if tg is None else fwAD.make_dual(out, t_out)
 
 
-# Normalise q inside the attention kernel where a kernel offers it (module switch for A/B timing and tests).
+# Normalise q / q and k inside the attention kernel where a kernel offers it (module switches for A/B timing and tests).
 IN_KERNEL_Q_NORM = True
+IN_KERNEL_K_NORM = True
+# A work-group of the tuned kernels covers 256 query rows and normalises the key tiles it consumes, so beyond that
+# length a head's keys would be normalised once per query block: measured slower than one stand-alone pass over k
+# (47.2 vs 46.7 ms on the DMFT-XL/2 512px forward+JVP step), so longer sequences keep that pass.
+K_NORM_IN_KERNEL_MAX_LQ = 256
 
 
 class QKNormAttnQKVPackedFunc(torch.autograd.Function):
     """(qkv, tqkv, q_gain, k_gain, eps, softmax_scale) -> (o, lse, to): per-head RMS
     norm of the q and k slots of a packed (B, L, 3, H, D) projection output followed
     by attention -- ``q, k = self.q_norm(q), self.k_norm(k); x = self.attn(q, k, v)``
-    (reference models/layers.py:147-151) -- as one autograd node.  Forward is the
-    fused RMS-norm kernel (primal + tangent) on the k slot, read in place, then the
-    attention kernel, which normalises q (and its tangent) itself while loading it;
-    where no kernel offers that (fp32, untuned shapes) the q slot goes through the
-    RMS-norm kernel as well.  Backward sends dv and the two norm gradients straight
-    into the three slots of one packed gradient buffer.  ``qn`` is None when q was
-    normalised inside the attention kernel (backward then recomputes it)."""
+    (reference models/layers.py:147-151) -- as one autograd node.  Forward is ONE
+    launch where a tuned kernel exists: the attention kernel reads the raw q, k, v
+    slots in place, normalises q (and its tangent) while loading it and every key
+    tile once it sits in on-chip memory, and hands the normalised primal rows to
+    the backward pass as two extra outputs.  Otherwise (fp32, untuned shapes, or the
+    module switches above) the k slot / both slots go through the stand-alone
+    RMS-norm kernel first.  Backward sends dv and the two norm gradients straight
+    into the three slots of one packed gradient buffer.  ``qn`` is None only when q
+    was normalised inside the kernel without being saved (backward then recomputes it)."""
 
     @staticmethod
     def forward(qkv, tqkv, q_gain, k_gain, eps, softmax_scale):
@@ -272,11 +279,18 @@ class QKNormAttnQKVPackedFunc(torch.autograd.Function):
         scale = _default_scale(q, softmax_scale)
         jvp = tqkv is not None
         tq, tk, tv = tqkv.unbind(2) if jvp else (None, None, None)
+        # the normalised rows are written only when a backward pass can follow
+        save = any(isinstance(t, torch.Tensor) and t.requires_grad for t in (qkv, q_gain, k_gain))
+        if IN_KERNEL_Q_NORM and IN_KERNEL_K_NORM and q.shape[1] <= K_NORM_IN_KERNEL_MAX_LQ:
+            fused = _lib.fwd_qknorm(q, k, v, tq, tk, tv, q_gain, k_gain, eps, scale, save_normed=save)
+            if fused is not None:
+                o, to, lse, qn, kn = fused
+                return o, lse, to, qn, kn
         kn, tkn = _lib.rmsnorm_fwd(k, k_gain, tk, eps, jvp)
-        fused = _lib.fwd_qnorm(q, kn, v, tq, tkn, tv, q_gain, eps, scale) if IN_KERNEL_Q_NORM else None
+        fused = _lib.fwd_qknorm(q, kn, v, tq, tkn, tv, q_gain, None, eps, scale, save_normed=save) if IN_KERNEL_Q_NORM else None
         if fused is not None:
-            o, to, lse = fused
-            return o, lse, to, None, kn
+            o, to, lse, qn, _ = fused
+            return o, lse, to, qn, kn
         qn, tqn = _lib.rmsnorm_fwd(q, q_gain, tq, eps, jvp)
         if jvp:
             o, to, lse = _lib.fwd_jvp(qn, kn, v, tqn, tkn, tv, scale)
@@ -300,8 +314,10 @@ class QKNormAttnQKVPackedFunc(torch.autograd.Function):
             return (None,) * 6
         qkv, q_gain, k_gain, qn, kn, o, lse = ctx.saved_tensors
         q, k, v = qkv.unbind(2)
-        if qn is None:
+        if qn is None:   # normalised in the kernel without being saved (no input asked for a gradient at forward time)
             qn, _ = _lib.rmsnorm_fwd(q, q_gain, None, ctx.eps, False)
+        if kn is None:
+            kn, _ = _lib.rmsnorm_fwd(k, k_gain, None, ctx.eps, False)
         gqkv = torch.empty(qkv.shape, dtype=qkv.dtype, device=qkv.device)
         gq, gk, gv = gqkv.unbind(2)
         dqn = torch.empty(qn.shape, dtype=qn.dtype, device=qn.device)
@@ -322,6 +338,10 @@ def flash_attn_qknorm_qkvpacked_func(qkv, q_gain, k_gain, eps: float = 1e-6, sof
     if tg is None and _lib.plain_inference(p, q_gain, k_gain):
         q, k, v = p.unbind(2)
         scale = _default_scale(q, softmax_scale)
+        if IN_KERNEL_Q_NORM and IN_KERNEL_K_NORM and q.shape[1] <= K_NORM_IN_KERNEL_MAX_LQ:
+            fused = _lib.fwd_qknorm(q, k, v, None, None, None, q_gain, k_gain, eps, scale, need_lse=False)
+            if fused is not None:
+                return fused[0]
         kn, _ = _lib.rmsnorm_fwd(k, k_gain, None, eps, False)
         fused = _lib.fwd_qnorm(q, kn, v, None, None, None, q_gain, eps, scale, need_lse=False) if IN_KERNEL_Q_NORM else None
         if fused is not None:

@@ -287,6 +287,7 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     all_cases = [("DMFT-B/2", "DMFT-B/2", 64, 8, "jvp", 32, False), ("DMFT-XL/2", "DMFT-XL/2", 32, 20, "train", 32, False),
                  ("DMFT-B/2 no-grad", "DMFT-B/2", 128, 8, "nograd", 32, False),
                  ("DMFT-XL/2 512px qk-norm", "DMFT-XL/2", 16, 20, "jvp", 64, True),
+                 ("DMFT-XL/2 512px qk-norm train", "DMFT-XL/2", 8, 20, "train", 64, True),
                  ("DMFT-XL/2 DMF loss step (mg)", "DMFT-XL/2", 16, 20, "dmf_loss", 32, False),
                  ("SiT-XL/2 FM train step", "SiT-XL/2", 32, None, "fm", 32, False),
                  ("DMFT-XL/2 4-step sampling cfg 1.5", "DMFT-XL/2", 64, 20, "sample", 32, False)]

@@ -124,6 +124,31 @@ DMF_ATTN_API int dmf_attn_fwd_qnorm(const void* q, const void* k, const void* v,
                      float scale, int dtype, void* stream);
 
 /*
+ * The same with the per-head RMS norm of k folded in as well -- the whole of
+ * `q, k = self.q_norm(q), self.k_norm(k); x = self.attn(q, k, v)`
+ * (models/layers.py:147-151) as one launch on the raw projections.  Every key
+ * tile is normalised (primal and tangent, same formulas with k_gain and the same
+ * eps, rounded to `dtype`) in on-chip memory between its arrival and its use;
+ * a work-group does this for the tiles it consumes, so a head's keys are
+ * normalised once per 256 query rows.
+ * q_hat, k_hat: optional contiguous (B, L, H, D) outputs of `dtype` (16-byte
+ * aligned) that receive the normalised primal rows -- what dmf_attn_bwd and
+ * dmf_rmsnorm_bwd need later -- or NULL when no backward pass follows.
+ * k_gain == NULL: k is read as given (already normalised) and k_hat is ignored,
+ * i.e. dmf_attn_fwd_qnorm with the q_hat output.
+ * Same strides table, optional arguments and DMF_ATTN_ENOKERNEL behaviour as
+ * dmf_attn_fwd_qnorm.
+ */
+DMF_ATTN_API int dmf_attn_fwd_qknorm(const void* q, const void* k, const void* v,
+                     const void* tq, const void* tk, const void* tv,
+                     const float* q_gain, const float* k_gain, float eps,
+                     void* o, void* to, float* lse, float* dlse,
+                     void* q_hat, void* k_hat,
+                     const int64_t* strides,
+                     int B, int H, int Lq, int Lkv, int D,
+                     float scale, int dtype, void* stream);
+
+/*
  * Backward on the primal output: dQ, dK, dV from (dout, q, k, v, o, lse).
  * Replaces `flash_attn_2_cuda.bwd` as called at
  * models/flash_attention_2_jvp.py:262-275.  Deterministic (no atomics).

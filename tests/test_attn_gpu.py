@@ -476,6 +476,100 @@ def test_qknorm_qkvpacked_in_kernel_q_norm():
         assert torch.equal(dmf_amd.flash_attn_qknorm_qkvpacked_func(qkv, gq, gk), o1.detach())
 
 
+@pytest.mark.parametrize("jvp", [True, False])
+@pytest.mark.parametrize("shape", QNORM_SHAPES)
+def test_fwd_qknorm_matches_separate_norms_and_oracle(shape, jvp):
+    """q AND k normalised inside the attention kernel (one launch on the raw projections) against (a) the separate
+    RMS-norm kernel on both followed by the plain attention kernel -- the key tiles are normalised with that kernel's
+    arithmetic element for element, so k_hat must carry the same bits; q_hat differs through the order of the sum of
+    squares only -- and (b) the fp32 oracle: restated RMSNorm.forward (models/layers.py:39-42, 147-151), its tangent
+    by torch.func.jvp, naive attention."""
+    from oracle import block_oracle as bo
+    B, Lq, Lkv, H, D = shape
+    g = torch.Generator().manual_seed(211 + D + Lq)
+    mk = lambda L: torch.randn(B, L, H, D, generator=g).to(torch.bfloat16)
+    q, tq, k, tk, v, tv = mk(Lq), mk(Lq), mk(Lkv), mk(Lkv), mk(Lkv), mk(Lkv)
+    q = q * (0.25 + 4 * torch.rand(B, Lq, H, 1, generator=g)).to(torch.bfloat16)   # rows of very different norms
+    k = k * (0.25 + 4 * torch.rand(B, Lkv, H, 1, generator=g)).to(torch.bfloat16)
+    gq, gk = 1 + 0.3 * torch.randn(D, generator=g), 1 + 0.3 * torch.randn(D, generator=g)
+    eps, scale = 1e-6, D ** -0.5
+    d = lambda t: t.to(DEV)
+    tang = (d(tq), d(tk), d(tv)) if jvp else (None, None, None)
+    got = _lib.fwd_qknorm(d(q), d(k), d(v), *tang, d(gq), d(gk), eps, scale, save_normed=True)
+    assert got is not None, "the tuned bf16 kernels cover every shape in this list"
+    o, to, lse, qh, kh = got
+    lean = _lib.fwd_qknorm(d(q), d(k), d(v), *tang, d(gq), d(gk), eps, scale, save_normed=False)
+    assert lean[3] is None and lean[4] is None and torch.equal(lean[0], o) and torch.equal(lean[2], lse)
+    qn, tqn = _lib.rmsnorm_fwd(d(q), d(gq), d(tq) if jvp else None, eps, jvp)
+    kn, tkn = _lib.rmsnorm_fwd(d(k), d(gk), d(tk) if jvp else None, eps, jvp)
+    assert torch.equal(kh, kn)
+    assert ao.rel_l2(qh.float(), qn.float()) <= 3e-3
+    if jvp:
+        o2, to2, lse2 = _lib.fwd_jvp(qn, kn, d(v), tqn, tkn, d(tv), scale)
+        assert ao.rel_l2(to.float(), to2.float()) <= 3e-3
+    else:
+        o2, lse2 = _lib.fwd(qn, kn, d(v), scale)
+        assert to is None
+    assert ao.rel_l2(o.float(), o2.float()) <= 3e-3 and ao.rel_l2(lse, lse2) <= 1e-3
+    f = lambda t: t.float()
+    if jvp:
+        (qn_ref, kn_ref), (tqn_ref, tkn_ref) = bo.jvp(lambda x, y: (bo.rms_norm(x, gq, eps), bo.rms_norm(y, gk, eps)), (f(q), f(k)), (f(tq), f(tk)))
+        o_ref, to_ref = ao.base_attn_jvp(qn_ref, kn_ref, f(v), tqn_ref, tkn_ref, f(tv))
+        assert ao.rel_l2(to.float().cpu(), to_ref) <= TOL[torch.bfloat16]
+    else:
+        o_ref = ao.base_attn(bo.rms_norm(f(q), gq, eps), bo.rms_norm(f(k), gk, eps), f(v))
+    assert ao.rel_l2(o.float().cpu(), o_ref) <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("L", [264, 1024, 256, 77])
+def test_qknorm_qkvpacked_in_kernel_norms_forward_and_backward_vs_oracle(L, monkeypatch):
+    """The packed q/k-norm + attention node on the tuned path.  Up to 256 rows the forward is ONE attention launch on
+    the raw projections; beyond, k takes one stand-alone RMS-norm pass (a head's keys would otherwise be normalised
+    once per 256-row query block) and q is still normalised in the kernel.  q never goes through the stand-alone
+    kernel, neither in the forward nor as a recompute in the backward.  Output, tangent and every gradient -- packed
+    qkv and both gains -- agree with autograd / forward-mode AD through the fp32 oracle (restated RMSNorm + naive
+    attention) on the CPU."""
+    import dmf_amd
+    from oracle import block_oracle as bo
+    B, H, D = 2, 3, 72
+    g = torch.Generator().manual_seed(31 + L)
+    qkv = torch.randn(B, L, 3, H, D, generator=g).to(torch.bfloat16)
+    tqkv = torch.randn(B, L, 3, H, D, generator=g).to(torch.bfloat16)
+    dout = torch.randn(B, L, H, D, generator=g).to(torch.bfloat16)
+    gq0, gk0 = 1 + 0.2 * torch.randn(D, generator=g), 1 + 0.2 * torch.randn(D, generator=g)
+    gq, gk = gq0.to(DEV).requires_grad_(), gk0.to(DEV).requires_grad_()
+    a = qkv.to(DEV).requires_grad_()
+
+    real, calls = _lib.rmsnorm_fwd, []
+
+    def counted(x, gain, *args, **kw):
+        calls.append(x.data_ptr())
+        return real(x, gain, *args, **kw)
+    monkeypatch.setattr(_lib, "rmsnorm_fwd", counted)
+    o, to = torch.func.jvp(lambda x: dmf_amd.flash_attn_qknorm_qkvpacked_func(x, gq, gk), (a,), (tqkv.to(DEV),))
+    k_slot = a.detach().unbind(2)[1].data_ptr()
+    assert calls == ([] if L <= 256 else [k_slot]), "stand-alone norm launches in the forward"
+    o.backward(dout.to(DEV))
+    assert len(calls) == (0 if L <= 256 else 1), "the backward must not re-normalise anything"
+    with torch.no_grad():
+        assert ao.rel_l2(dmf_amd.flash_attn_qknorm_qkvpacked_func(qkv.to(DEV), gq, gk).float(), o.detach().float()) <= 1e-6
+    monkeypatch.undo()
+
+    x = qkv.float().requires_grad_()
+    rq, rk = gq0.clone().requires_grad_(), gk0.clone().requires_grad_()
+
+    def ref(x_):
+        q, k, v = x_.unbind(2)
+        return ao.base_attn(bo.rms_norm(q, rq, 1e-6), bo.rms_norm(k, rk, 1e-6), v)
+
+    o_ref, to_ref = torch.func.jvp(ref, (x,), (tqkv.float(),))
+    o_ref.backward(dout.float())
+    tol = TOL[torch.bfloat16]
+    r = lambda got, exp: ao.rel_l2(got.detach().float().cpu(), exp.detach())
+    assert r(o, o_ref) <= tol and r(to, to_ref) <= tol
+    assert r(a.grad, x.grad) <= tol and r(gq.grad, rq.grad) <= tol and r(gk.grad, rk.grad) <= tol
+
+
 def test_golden_vectors():
     """fp32 kernels through the C ABI against the committed known-answer vectors
     (tests/golden/attn_vectors.npz: fp64 closed forms on seeded inputs, one case with Lq != Lkv)."""
