@@ -29,7 +29,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = _declared_symbols()
-    assert len(names) == 20 and set(names) == set(_lib.SIGNATURES), names
+    assert len(names) == 21 and set(names) == set(_lib.SIGNATURES), names
     for n in names:
         assert getattr(lib, n) is not None
     assert lib.dmf_attn_version() >= 1
