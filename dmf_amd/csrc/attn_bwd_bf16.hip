@@ -497,24 +497,33 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
   if (tid < 256) stat_lse[tid] = tid < p.Lq ? p.lse[(int64_t)bh * p.Lq + tid] : INFINITY;   // +inf switches padded query rows off (P = 0)
   DeltaRows dr = delta_request(0);
   issue_q(0);
-  // ---- this lane's key row: K (times scale*log2e) and V stay in registers
-  const int krow = wave * 32 + c32;
-  u32x4 Kr[NCHUNK], Vr[NCHUNK];
-  load_row_chunks<NCHUNK, VPR>(rs_k, rb_k, krow, g, Kr);
-  load_row_chunks<NCHUNK, VPR>(rs_v, rb_v, krow, g, Vr);
+  // ---- this wave's 32 key rows, whole rows by DMA: K straight into its tile of the LDS-resident copy (the phase 2
+  //      operand, and where phase 1 takes its register operand from), V into the exchange area, which nobody uses
+  //      before the first barrier (rows past Lkv read as zeros)
+  issue_rows<P, VPR, 32>(rs_k, rb_k, (uint32_t)(wave * 32) * rb_k, smem + FC::K_OFF + wave * TB, lane);
+  issue_rows<P, VPR, 32>(rs_v, rb_v, (uint32_t)(wave * 32) * rb_v, smem + FC::X_OFF + wave * TB, lane);
   for (int j = 1; j < NST - 1 && j < nqt; ++j) issue_q(j);
-  // the LDS-resident copy of K (phase 2 operand) comes from these registers rather than from a second trip to memory:
-  // lane (c32, g) holds vectors 2c + g of row krow (rows past Lkv were read as zeros)
+  wait_tile(0);   // loads complete in order: the key rows (and tile 0) have landed, the later tiles may still be in flight
+  // ---- this lane's key row: V stays in registers for the whole kernel, K (times scale*log2e) is re-read from the LDS
+  //      copy at the top of every half (so that its registers are free while dQ is formed)
+  const int krow = wave * 32 + c32;
+  const uint32_t k_row_addr = lds_addr(smem) + FC::K_OFF + (krow * P + g) * 16;   // pad vectors of the K tiles are zero
+  u32x4 Kr[NCHUNK], Vr[NCHUNK];
   {
-    const uint32_t ka = lds_addr(smem) + FC::K_OFF + (krow * P + g) * 16;
+    const uint32_t va = lds_addr(smem) + FC::X_OFF + krow * P * 16;
     static_for<NCHUNK>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
-      if (2 * c + g < VPR) lds_write128_untracked<32 * c>(ka, Kr[c]);
+      // (the upper half of the last chunk of a head dim that is not a multiple of 16 does not exist: zeroed below)
+      Vr[c] = lds_read128_issue<32 * c>(2 * c + 1 < VPR ? va + g * 16 : va);
     });
+    lds_read128_wait<0>(Vr[NCHUNK - 1]);
+#pragma unroll
+    for (int c = 0; c + 1 < NCHUNK; ++c) asm volatile("" : "+v"(Vr[c]));
+    if constexpr (2 * NCHUNK > VPR) {
+      if (g == 1) Vr[NCHUNK - 1] = u32x4{0, 0, 0, 0};
+    }
   }
   delta_finish(0, dr);
-#pragma unroll
-  for (int c = 0; c < NCHUNK; ++c) Kr[c] = scale_bf16x8(Kr[c], p.scale_log2);
   const bool kvalid = krow < p.Lkv;
 
   f32x16 dK[NMT], dV[NMT];
@@ -538,10 +547,15 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
   for (int half = 0; half * 4 < nqt; ++half) {
     // ================= phase 1: query tiles 4*half .. 4*half+3 against this wave's keys
     const int j_end = min(nqt, 4 * half + 4);
+    static_for<NCHUNK>([&](auto cc) { Kr[decltype(cc)::value] = lds_read128_issue<32 * decltype(cc)::value>(k_row_addr); });
+    lds_read128_wait<0>(Kr[NCHUNK - 1]);
+#pragma unroll
+    for (int c = 0; c + 1 < NCHUNK; ++c) asm volatile("" : "+v"(Kr[c]));
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) Kr[c] = scale_bf16x8(Kr[c], p.scale_log2);
     for (int j = 4 * half; j < j_end; ++j) {
       if (j == 0 || j != 4 * half) {   // (the first tile of a later half was waited for before the dQ rows were stored)
         wait_tile(j);     // this wave's share of tile j has landed
-        if (j == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and its rows of the K copy are in LDS
         lds_barrier();    // ... and everyone else's; all waves are done with the stage of tile j-1
       }
       if (j + 1 < nqt) dr = delta_request(j + 1);   // (before the tile request: its data is wanted first)
@@ -658,31 +672,74 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
       };
       const T* kt = reinterpret_cast<const T*>(smem + FC::K_OFF);
       constexpr int NT1 = NMT - NT0;
-      for (int kb = 0; kb < nkb; ++kb, xt += FC::XTILE / 2, kt += TB / 2) {
-        // B operands: dS^T of 16 keys each (steps 0, 1) for this wave's 32 queries; A operands: K^T tiles of this part
-        const ColOperand b0 = x_operand(xt, 0), b1 = x_operand(xt, 1);
+      // Operands of one key block: dS^T of 16 keys each (steps 0, 1) for this wave's 32 queries (B), the K^T tiles of this
+      // wave's part (A).  The operands of block kb + 1 are requested before the products of block kb are issued, so
+      // that only the first block waits for the LDS.
+      struct Ops { ColOperand b0, b1, a0, a1, a2, a3, tail; };   // (plain members: an array member ends up in scratch memory)
+      static_assert(NT0 <= 2 && NT1 <= 2, "operand slots for at most two output tiles per part");
+      auto load_ops = [&](int kb, Ops& o) {
+        const T* x = xt + kb * (FC::XTILE / 2);
+        const T* kk = kt + kb * (TB / 2);
+        o.b0 = x_operand(x, 0);
+        o.b1 = x_operand(x, 1);
+        auto tile_ops = [&](int col, ColOperand& s0, ColOperand& s1) {
+          s0 = lds_col_operand<T, STR>(kk, 0, col, 0, lane);
+          s1 = lds_col_operand<T, STR>(kk, 0, col, 1, lane);
+        };
         if (!part1) {
-          static_for<NT0>([&](auto tc) {
-            constexpr int t = decltype(tc)::value;
-            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * t, 0, lane), b0);
-            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * t, 1, lane), b1);
-          });
+          tile_ops(0, o.a0, o.a1);
+          if constexpr (NT0 > 1) tile_ops(32, o.a2, o.a3);
           if constexpr (TAIL) {
-            const T* tp = kt + tail_lane_offset(lane, STR, 32 * NMT);
+            const T* tp = kk + tail_lane_offset(lane, STR, 32 * NMT);
             const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, tp)));
             const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, tp + 8 * STR)));
-            ColOperand ka, d0, d1;
-            ka.v = u32x4{lo[0], lo[1], hi[0], hi[1]};
-            tail_operands(b0, b1, d0, d1);
-            mma16(dQ16[0], ka, d0);
-            mma16(dQ16[1], ka, d1);
+            o.tail.v = u32x4{lo[0], lo[1], hi[0], hi[1]};
           }
         } else {
-          static_for<NT1>([&](auto tc) {
-            constexpr int t = decltype(tc)::value;
-            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * (NT0 + t), 0, lane), b0);
-            mma_col<T>(dQ[t], lds_col_operand<T, STR>(kt, 0, 32 * (NT0 + t), 1, lane), b1);
-          });
+          if constexpr (NT1 > 0) tile_ops(32 * NT0, o.a0, o.a1);
+          if constexpr (NT1 > 1) tile_ops(32 * (NT0 + 1), o.a2, o.a3);
+        }
+      };
+      auto multiply = [&](const Ops& o) {
+        if (!part1) {
+          mma_col<T>(dQ[0], o.a0, o.b0);
+          mma_col<T>(dQ[0], o.a1, o.b1);
+          if constexpr (NT0 > 1) {
+            mma_col<T>(dQ[1], o.a2, o.b0);
+            mma_col<T>(dQ[1], o.a3, o.b1);
+          }
+          if constexpr (TAIL) {
+            ColOperand d0, d1;
+            tail_operands(o.b0, o.b1, d0, d1);
+            mma16(dQ16[0], o.tail, d0);
+            mma16(dQ16[1], o.tail, d1);
+          }
+        } else {
+          if constexpr (NT1 > 0) {
+            mma_col<T>(dQ[0], o.a0, o.b0);
+            mma_col<T>(dQ[0], o.a1, o.b1);
+          }
+          if constexpr (NT1 > 1) {
+            mma_col<T>(dQ[1], o.a2, o.b0);
+            mma_col<T>(dQ[1], o.a3, o.b1);
+          }
+        }
+      };
+      Ops oa, ob;
+      if constexpr (NMT <= 2) {
+        load_ops(0, oa);
+        for (int kb = 0; kb < nkb; kb += 2) {
+          if (kb + 1 < nkb) load_ops(kb + 1, ob);
+          multiply(oa);
+          if (kb + 1 < nkb) {
+            if (kb + 2 < nkb) load_ops(kb + 2, oa);
+            multiply(ob);
+          }
+        }
+      } else {   // three output tiles: no registers left for a second operand set
+        for (int kb = 0; kb < nkb; ++kb) {
+          load_ops(kb, oa);
+          multiply(oa);
         }
       }
     }
