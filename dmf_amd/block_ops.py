@@ -39,6 +39,17 @@ def _unpack(*tensors):
     return primals, tangents, any(tg is not None for tg in tangents)
 
 
+def _primal_only(*tangent_cotangents):
+    """These operators differentiate through their primal output only.  A loss that keeps the JVP output attached
+    (unlike the MeanFlow loss, loss.py:171-172) would need the second-order terms the reference's tensor expressions
+    carry; say so instead of returning gradients that silently lack them."""
+    if any(g is not None for g in tangent_cotangents):
+        raise NotImplementedError(
+            "dmf_amd.block_ops: a gradient arrived at the tangent (JVP) output of a fused block operator; these operators "
+            "back-propagate through the primal output only -- detach the JVP output (as DMFLoss does) or build the model "
+            "with block_ops='torch'")
+
+
 def _like(g, ref):
     """Gradient of a (B, C) modulation operand reshaped to the operand's shape."""
     return g.reshape(ref)
@@ -60,6 +71,7 @@ class LNModulateFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gty):
+        _primal_only(gty)
         if gy is None:
             return (None,) * 9
         x, scale = ctx.saved_tensors
@@ -83,6 +95,7 @@ class GateResidualFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gty):
+        _primal_only(gty)
         if gy is None:
             return (None,) * 7
         gate, h = ctx.saved_tensors
@@ -106,6 +119,7 @@ class ResidualLNModulateFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gz, gty, gtz):
+        _primal_only(gty, gtz)
         if gy is None and gz is None:
             return (None,) * 13
         y, h, gate, scale = ctx.saved_tensors
@@ -130,6 +144,7 @@ class GeluTanhFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gty):
+        _primal_only(gty)
         if gy is None:
             return None, None
         (x,) = ctx.saved_tensors
@@ -150,6 +165,7 @@ class SiluFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gty):
+        _primal_only(gty)
         if gy is None:
             return None, None, None
         (x,) = ctx.saved_tensors
@@ -172,6 +188,7 @@ class RMSNormFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gty):
+        _primal_only(gty)
         if gy is None:
             return (None,) * 5
         x, gain = ctx.saved_tensors
@@ -220,6 +237,7 @@ class DualLinearFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gty, gw_unused):
+        _primal_only(gty)
         if gy is None:
             return (None,) * 6
         x, w = ctx.saved_tensors
@@ -246,7 +264,13 @@ class DualLinearFunc(torch.autograd.Function):
             if want_gb:
                 # torch's multi-block column reduction clears its scratch with a memset node, which does not survive
                 # HIP-graph replay; the library's two-stage sum has no such node
-                gb = _lib.colsum(g2.contiguous(), ctx.bias_dtype) if g2.is_cuda and g2.shape[1] % 8 == 0 else g2.sum(0).to(ctx.bias_dtype)
+                if g2.is_cuda and g2.shape[1] % 8 == 0:
+                    gb = _lib.colsum(g2.contiguous(), ctx.bias_dtype)
+                else:
+                    if g2.is_cuda and torch.cuda.is_current_stream_capturing():
+                        raise RuntimeError("dual_linear: the bias gradient of a layer whose output width is not a multiple of 8 falls back "
+                                           "to torch's column sum, which does not replay correctly from a captured graph")
+                    gb = g2.sum(0).to(ctx.bias_dtype)
         finally:
             if fork:
                 torch.cuda.set_stream(main)

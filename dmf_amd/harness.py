@@ -212,6 +212,19 @@ def build_model(name: str, attn_func: str, device, qk_norm: bool = False, input_
     return model.init_trunc_normal_(0.02, seed)
 
 
+def stale_grad_accumulator(p: torch.Tensor) -> bool:
+    """True if an autograd graph that is still alive refers to ``p``'s gradient accumulator.  The accumulator node is
+    created on first use and freed with the last graph that points at it; asking for it twice returns the same
+    object only while something else keeps it alive."""
+    key = "dmf_amd.stale_probe"
+    node = p.view_as(p).grad_fn.next_functions[0][0]
+    node.metadata[key] = True          # lives on the node itself, not on this Python wrapper
+    del node
+    node = p.view_as(p).grad_fn.next_functions[0][0]
+    alive = bool(node.metadata.pop(key, False))
+    return alive
+
+
 class GraphedStep:
     """A step function captured once into a HIP graph and replayed.
 
@@ -221,17 +234,25 @@ class GraphedStep:
     a captured graph removes the host from the loop.  ``fn(*inputs)`` must be a
     pure function of its tensor arguments (and of module parameters, which are
     read in place at replay time); its outputs live in the graph's memory pool
-    and are overwritten by the next call.  Capture happens on a side stream at
-    the default priority after ``warmup`` eager calls.  If ``fn`` runs a backward
-    pass, no autograd graph of an earlier step may be alive when the step is
-    captured (keep ``float(loss)`` or ``loss.detach()``, not ``loss``): a parameter's
-    gradient accumulator lives as long as any graph refers to it and stays bound to
-    the stream it was created on, so the captured backward would be sent to a stream
-    that is not capturing, which the runtime answers with a crash, not an error.
+    and are overwritten by the next call.  The ``warmup`` eager calls and the
+    capture run on ONE side stream at the default priority: a parameter's gradient
+    accumulator is bound to the stream it was created on, so the accumulators
+    that the warm-up creates are the ones the captured backward uses.  What the
+    class cannot see is an autograd graph of an EARLIER step that the caller still
+    holds (``loss`` kept instead of ``float(loss)`` / ``loss.detach()``): it keeps
+    older accumulators alive, bound to the caller's stream, and the captured
+    backward would then be sent to a stream that is not capturing.  ``parameters``
+    (optional) lets the constructor refuse that case before capturing: it raises
+    if any of them still has a gradient accumulator from before the warm-up.
     """
 
-    def __init__(self, fn, *example_inputs, warmup: int = 3):
+    def __init__(self, fn, *example_inputs, warmup: int = 3, parameters=None):
         self.static_inputs = [x.clone() if isinstance(x, torch.Tensor) else x for x in example_inputs]
+        stale = [p for p in (parameters or ()) if p.requires_grad and stale_grad_accumulator(p)]
+        if stale:
+            raise RuntimeError(f"GraphedStep: {len(stale)} parameter(s) still have a gradient accumulator from an earlier step "
+                               "(an autograd graph of that step is alive: drop it, e.g. keep float(loss) instead of loss) -- a "
+                               "backward captured now would run on the stream that accumulator was created on")
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -240,7 +261,7 @@ class GraphedStep:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with torch.cuda.graph(self.graph, stream=side):
             self.static_outputs = fn(*self.static_inputs)
 
     def __call__(self, *inputs):
@@ -354,7 +375,7 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
             # the forward+JVP-only and no-grad passes run over frozen weights: cast them once, not per call
             frozen = frozen_low_precision_params(model) if (mode in ("jvp", "nograd") and block_ops == "hip") else contextlib.nullcontext()
             with frozen:
-                run = GraphedStep(step, *data) if graphed else step
+                run = GraphedStep(step, *data, parameters=list(model.parameters())) if graphed else step
                 sec = _time(lambda: run(*data), steps * 4 if graphed else (steps if op == "hip" else max(2, steps // 2)))
             row[f"{label}_ms_per_step"] = sec * 1e3
             row[f"{label}_images_per_s"] = batch / sec

@@ -80,3 +80,22 @@ def test_graphed_train_step_replays_match_eager():
             bad = [n for n, g in grads_ref.items() if not _same(params[n].grad, g)]
             assert not bad, f"replay {rep}: gradients differ from eager for {bad[:6]}"
             _eager_noise()
+
+
+def test_graphed_step_refuses_capture_while_an_earlier_graph_is_alive():
+    """A backward captured while an earlier step's autograd graph is alive would use gradient accumulators bound to
+    another stream (a runtime crash, not an error): the constructor refuses it on the host when it is given the parameters."""
+    model = harness.build_model("DMFT-B/2", "hip", DEV, dmf_depth=8, block_ops="hip")
+    batch = harness.synthetic_batch(2, DEV, seed=5)
+
+    def fn(z, t, r, y, v):
+        model.zero_grad(set_to_none=True)
+        return harness.train_step(model, (z, t, r, y, v)).detach()
+
+    kept = harness.train_step(model, batch)           # an attached loss: its graph stays alive
+    with pytest.raises(RuntimeError, match="gradient accumulator from an earlier step"):
+        harness.GraphedStep(fn, *batch, parameters=list(model.parameters()))
+    del kept
+    model.zero_grad(set_to_none=True)
+    step = harness.GraphedStep(fn, *batch, parameters=list(model.parameters()))
+    assert torch.isfinite(step(*batch)).all()

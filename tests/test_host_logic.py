@@ -296,3 +296,30 @@ def test_frozen_low_precision_params_nest_and_restore():
             assert m[0].lp_weight.dtype == torch.float16
         assert m[0].lp_weight is outer              # the inner context put the outer copies back
     assert m[0].lp_weight is None and m[0].lp_bias is None and m[1].lp_weight is None
+
+
+def test_fused_block_operators_refuse_a_gradient_at_their_tangent_output():
+    """The fused block operators back-propagate through the primal output only (exact for the MeanFlow loss, whose JVP
+    target is detached, loss.py:171-172).  A loss that keeps the JVP output attached must hear about it instead of
+    getting gradients without the second-order terms that the reference's tensor expressions would supply."""
+    from dmf_amd import block_ops
+    g = torch.ones(2, 3)
+    for fn, grads in ((block_ops.LNModulateFunc, (None, g)), (block_ops.GateResidualFunc, (g, g)),
+                      (block_ops.ResidualLNModulateFunc, (g, None, None, g)), (block_ops.GeluTanhFunc, (None, g)),
+                      (block_ops.SiluFunc, (g, g)), (block_ops.RMSNormFunc, (None, g)), (block_ops.DualLinearFunc, (g, g, None))):
+        with pytest.raises(NotImplementedError, match="primal output only"):
+            fn.backward(None, *grads)
+
+
+def test_stale_gradient_accumulator_probe():
+    """GraphedStep refuses to capture a backward pass while an autograd graph of an earlier step is alive; the probe
+    behind that refusal, on the CPU."""
+    from dmf_amd.harness import stale_grad_accumulator
+    p = torch.nn.Parameter(torch.randn(3))
+    assert not stale_grad_accumulator(p) and not stale_grad_accumulator(p)
+    loss = (p * 2).sum()
+    assert stale_grad_accumulator(p)
+    loss.backward()
+    assert stale_grad_accumulator(p)          # the graph's nodes live as long as `loss` does
+    del loss
+    assert not stale_grad_accumulator(p)
