@@ -563,83 +563,132 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
       const uint32_t stage_off = FC::QS_OFF + (j % NST) * STAGE;
       const uint32_t ra = row_addr + stage_off, ca = lds_addr(smem) + col_off + stage_off;
 
-      // ---- S = Q K^T (log2 units), dP = dout V^T : rows = queries (in-lane), columns = keys (lanes)
-      f32x16 S = {0}, dP = {0};
+      // ---- The four products of a tile are four MFMA runs: S = Q K^T (log2 units) and dP = dout V^T (rows = queries,
+      //      in-lane; columns = keys, lanes), then dV^T += dout^T P and dK^T += Q^T dS.  The arithmetic in between is issued
+      //      inside the run that does not depend on it -- P = exp2(S - lse*log2e) between the MFMAs of dP, dS = P (dP - delta)
+      //      and its hand-over to the exchange array between the MFMAs of dV -- because an MFMA holds the matrix pipe for 32
+      //      cycles but the issue port for 4, and a wave issues in order: only interleaved in program order do the two overlap
+      //      (left alone the scheduler gathers the MFMAs, hence the pins).  Padded query rows carry lse = +inf (P = 0), padded
+      //      keys are switched off where dS is handed over.
+#define DMF_PIN() __builtin_amdgcn_sched_barrier(0)
+      f32x16 S = {0}, dP = {0}, Pm, dS;
+      ColOperand pp[2], ds[2];
+      const uint32_t xa = x_base + ((j & 3) * 8 + wave) * FC::XTILE + c32 * 64;   // this lane's key row of tile X[j % 4][wave]
+      // lse / delta of the slice's four queries: raw reads like the operands, requested one slice ahead (a tracked read
+      // would be waited for with lgkmcnt(0), i.e. together with the operand reads just issued behind it)
+      const uint32_t stat_addr = lds_addr(stat_lse) + (j * 32 + 4 * g) * 4;
+      u32x4 sl[2], sd[2];
+      auto p_slice = [&](auto jc) {   // elements 4jj .. 4jj+3: queries 8jj + 4g .. +3 of the tile
+        constexpr int jj = decltype(jc)::value;
+        const u32x4 l4 = sl[jj & 1];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) Pm[4 * jj + e] = fast_exp2(fmaf(__uint_as_float(l4[e]), -kLog2e, S[4 * jj + e]));
+        if constexpr (jj & 1) pp[jj >> 1] = acc_operand<T>(Pm, jj >> 1);
+      };
+      auto ds_slice = [&](auto jc) {
+        constexpr int jj = decltype(jc)::value;
+        const u32x4 d4 = sd[jj & 1];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dS[4 * jj + e] = Pm[4 * jj + e] * (dP[4 * jj + e] - __uint_as_float(d4[e]));
+        if constexpr (jj & 1) {
+          ds[jj >> 1] = acc_operand<T>(dS, jj >> 1);
+          // dS tile -> X (zeros for keys past the end: their K rows must not reach dQ)
+          static_for<2>([&](auto hc) {
+            constexpr int q4 = jj - 1 + decltype(hc)::value;   // queries 8 q4 + 4g .. +3 of key row c32
+            const u32x2 w = kvalid ? u32x2{ds[q4 >> 1].v[2 * (q4 & 1)], ds[q4 >> 1].v[2 * (q4 & 1) + 1]} : u32x2{0, 0};
+            lds_write64_untracked<0>(xa + (((2 * q4 + g) ^ x_swz) << 3), w);
+          });
+        }
+      };
+      static_assert(NCHUNK >= 4, "the four P slices ride between the first four dP MFMAs");
       {
         u32x4 qc[2], oc[2];
         qc[0] = lds_read128_issue<0>(ra);
-        oc[0] = lds_read128_issue<DO_OFF>(ra);
-        static_for<NCHUNK>([&](auto cc) {
+        static_for<NCHUNK>([&](auto cc) {   // run 1: S
+          constexpr int c = decltype(cc)::value;
+          if constexpr (c + 1 < NCHUNK) {
+            qc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
+            lds_read128_wait<1>(qc[c & 1]);
+          } else {   // first operand and first lse slice of the next run
+            oc[0] = lds_read128_issue<DO_OFF>(ra);
+            sl[0] = lds_read128_issue<0>(stat_addr);
+            lds_read128_wait<2>(qc[c & 1]);
+          }
+          mma_chunk<T>(S, qc[c & 1], Kr[c]);
+        });
+        static_for<NCHUNK>([&](auto cc) {   // run 2: dP, P formed meanwhile
           constexpr int c = decltype(cc)::value;
           constexpr bool more = c + 1 < NCHUNK;
-          if constexpr (more) {
-            qc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
-            oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
-          }
-          lds_read128_wait<more ? 2 : 0>(qc[c & 1], oc[c & 1]);
-          mma_chunk<T>(S, qc[c & 1], Kr[c]);
+          if constexpr (more) oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
+          if constexpr (c + 1 < 4) sl[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(stat_addr);   // 8 queries = 32 bytes per slice
+          // operand c and lse slice c were requested one step ago: leave what has been requested since in flight
+          if constexpr (c < 4) lds_read128_wait<(more ? 1 : 0) + (c + 1 < 4 ? 1 : 0)>(oc[c & 1], sl[c & 1]);
+          else lds_read128_wait<more ? 1 : 0>(oc[c & 1]);
+          DMF_PIN();
           mma_chunk<T>(dP, oc[c & 1], Vr[c]);
+          DMF_PIN();
+          if constexpr (c < 4) p_slice(cc);
+          DMF_PIN();
         });
       }
-      // ---- P = exp2(S - lse*log2e), dS = P * (dP - delta); padded query rows carry lse = +inf (P = 0), padded keys are
-      //      switched off below
-      f32x16 Pm, dS;
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(stat_lse + j * 32 + jj * 8 + 4 * g);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(stat_delta + j * 32 + jj * 8 + 4 * g);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 4 * jj + e;
-          Pm[i] = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
-          dS[i] = Pm[i] * (dP[i] - d4[e]);
-        }
-      }
-      ColOperand pp[2] = {acc_operand<T>(Pm, 0), acc_operand<T>(Pm, 1)};
-      ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
-      // ---- dS tile -> X[j % 4][wave] (zeros for keys past the end: their K rows must not reach dQ)
-      {
-        const uint32_t xa = x_base + ((j & 3) * 8 + wave) * FC::XTILE + c32 * 64;
-        static_for<4>([&](auto jc) {
-          constexpr int jj = decltype(jc)::value;
-          const u32x2 w = kvalid ? u32x2{ds[jj >> 1].v[2 * (jj & 1)], ds[jj >> 1].v[2 * (jj & 1) + 1]} : u32x2{0, 0};
-          lds_write64_untracked<0>(xa + (((2 * jj + g) ^ x_swz) << 3), w);   // queries 8jj + 4g .. +3 of key row c32
-        });
-      }
-      // ---- dV^T += dout^T P ; dK^T += Q^T dS
       {
         constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
+        static_assert(NGT >= 4, "the four dS slices ride between the first four dV MFMAs");
         TrPair qq[2], oo[2];
         auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
-        qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
+        const uint32_t ta = lds_addr(smem) + tail_off + stage_off;
         oo[0] = lds_tr16_issue<lo_off(0) + DO_OFF, lo_off(0) + 8 * STR * 2 + DO_OFF>(ca);
-        static_for<NGT>([&](auto gc) {
+        sd[0] = lds_read128_issue<1024>(stat_addr);   // stat_delta = stat_lse + 256 floats
+        static_for<NGT>([&](auto gc) {   // run 3: dV^T += dout^T P, dS formed and handed over meanwhile
+          constexpr int gi = decltype(gc)::value;
+          if constexpr (gi + 1 < NG) {
+            constexpr int LO = lo_off(gi + 1), HI = LO + 8 * STR * 2;
+            oo[(gi + 1) & 1] = lds_tr16_issue<LO + DO_OFF, HI + DO_OFF>(ca);
+          } else if constexpr (gi + 1 < NGT) {
+            oo[(gi + 1) & 1] = lds_tr16_issue<DO_OFF, 8 * STR * 2 + DO_OFF>(ta);
+          } else {
+            qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);   // first operand of the next run
+          }
+          if constexpr (gi + 1 < 4) sd[(gi + 1) & 1] = lds_read128_issue<1024 + 32 * (gi + 1)>(stat_addr);
+          if constexpr (gi < 4) {
+            asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(oo[gi & 1].lo), "+v"(oo[gi & 1].hi), "+v"(sd[gi & 1]) : [n] "n"(gi + 1 < 4 ? 3 : 2));
+          } else {
+            lds_tr16_wait<2>(oo[gi & 1]);
+          }
+          DMF_PIN();
+          if constexpr (gi < NG) {
+            mma_col<T>(dV[gi % NMT], tr_operand(oo[gi & 1]), pp[gi / NMT]);
+          } else {
+            ColOperand p0, p1;
+            tail_operands(pp[0], pp[1], p0, p1);
+            mma16(dV16[0], tr_operand(oo[gi & 1]), p0);
+            mma16(dV16[1], tr_operand(oo[gi & 1]), p1);
+          }
+          DMF_PIN();
+          if constexpr (gi < 4) ds_slice(gc);
+          DMF_PIN();
+        });
+        static_for<NGT>([&](auto gc) {   // run 4: dK^T += Q^T dS
           constexpr int gi = decltype(gc)::value;
           constexpr bool more = gi + 1 < NGT;
           if constexpr (gi + 1 < NG) {
             constexpr int LO = lo_off(gi + 1), HI = LO + 8 * STR * 2;
             qq[(gi + 1) & 1] = lds_tr16_issue<LO, HI>(ca);
-            oo[(gi + 1) & 1] = lds_tr16_issue<LO + DO_OFF, HI + DO_OFF>(ca);
           } else if constexpr (more) {
-            const uint32_t ta = lds_addr(smem) + tail_off + stage_off;
             qq[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(ta);
-            oo[(gi + 1) & 1] = lds_tr16_issue<DO_OFF, 8 * STR * 2 + DO_OFF>(ta);
           }
-          lds_tr16_wait<more ? 4 : 0>(qq[gi & 1], oo[gi & 1]);
+          lds_tr16_wait<more ? 2 : 0>(qq[gi & 1]);
           if constexpr (gi < NG) {
-            mma_col<T>(dV[gi % NMT], tr_operand(oo[gi & 1]), pp[gi / NMT]);
             mma_col<T>(dK[gi % NMT], tr_operand(qq[gi & 1]), ds[gi / NMT]);
           } else {
-            ColOperand p0, p1, d0, d1;
-            tail_operands(pp[0], pp[1], p0, p1);
+            ColOperand d0, d1;
             tail_operands(ds[0], ds[1], d0, d1);
-            mma16(dV16[0], tr_operand(oo[gi & 1]), p0);
-            mma16(dV16[1], tr_operand(oo[gi & 1]), p1);
             mma16(dK16[0], tr_operand(qq[gi & 1]), d0);
             mma16(dK16[1], tr_operand(qq[gi & 1]), d1);
           }
         });
       }
+#undef DMF_PIN
       if (j + 1 < nqt) delta_finish(j + 1, dr);   // visible to the other waves after the next barrier
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's dS tiles are in LDS
