@@ -36,8 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # `bench.py --workload W --kernel K` (each scaled by what the counter reads for a plain 1 GiB copy in the same run;
 # summaries in profiles/attn_<kernel>_bf16_d72_<workload>.txt).  The two-kernel backward at N=1024 reads q, k, v, dout twice.
 MEASURED_TRAFFIC_BYTES = {("fwd_jvp", "xl2_512px"): 1.2124e9, ("fwd_jvp", "xl2_256px"): 1.2123e9,
-                          ("fwd", "xl2_512px"): 6.0845e8, ("fwd", "xl2_256px"): 6.0906e8,
-                          ("bwd", "xl2_512px"): 1.8728e9, ("bwd", "xl2_256px"): 1.2170e9}
+                          ("fwd", "xl2_512px"): 6.0844e8, ("fwd", "xl2_256px"): 6.0936e8,
+                          ("bwd", "xl2_512px"): 1.8715e9, ("bwd", "xl2_256px"): 1.2838e9}
 
 DEVICE_WAKE_SECONDS = 0.3        # untimed launches of the measured kernel before the --warmup steps (clock ramp from idle)
 
@@ -165,8 +165,8 @@ PROFILE_FILES = {("fwd_jvp", "xl2_512px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_5
                  ("bwd", "xl2_512px"): "profiles/attn_bwd_bf16_d72_xl2_512px.txt", ("bwd", "xl2_256px"): "profiles/attn_bwd_bf16_d72_xl2_256px.txt"}
 # Share of the clocked cycles in which the MFMA pipe was busy (SQ_VALU_MFMA_BUSY_CYCLES / (4 SQ_BUSY_CU_CYCLES)), from the
 # rocprofv3 --pmc runs summarised in the files above (offline, like `traffic`); None where no such run is committed.
-MEASURED_MFMA_BUSY = {("fwd_jvp", "xl2_512px"): 0.588, ("fwd_jvp", "xl2_256px"): 0.363, ("fwd", "xl2_512px"): 0.492,
-                      ("fwd", "xl2_256px"): 0.294, ("bwd", "xl2_512px"): 0.436, ("bwd", "xl2_256px"): 0.189}
+MEASURED_MFMA_BUSY = {("fwd_jvp", "xl2_512px"): 0.585, ("fwd_jvp", "xl2_256px"): 0.354, ("fwd", "xl2_512px"): 0.491,
+                      ("fwd", "xl2_256px"): 0.277, ("bwd", "xl2_512px"): 0.436, ("bwd", "xl2_256px"): 0.195}
 
 
 def roofline(name, ms, kind="fwd_jvp"):
