@@ -157,7 +157,7 @@ def cpu_baseline_config1():
 
 
 # Kernels behind each entry point at the two workloads (rocprofv3 names), and where the offline counter figures live.
-KERNELS = {"fwd_jvp": "dmf::attn_fwd_bf16_kernel<72, true, 8, false>", "fwd": "dmf::attn_fwd_bf16_kernel<72, false, 8, false>",
+KERNELS = {"fwd_jvp": "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>", "fwd": "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>",
            "bwd": {"xl2_512px": "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72>",
                    "xl2_256px": "dmf::attn_bwd_fused_bf16_kernel<72>"}}
 PROFILE_FILES = {("fwd_jvp", "xl2_512px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_512px.txt", ("fwd_jvp", "xl2_256px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_256px.txt",
