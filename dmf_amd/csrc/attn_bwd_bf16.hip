@@ -15,6 +15,9 @@
 #define DMF_BWD_FUSED 1   // 0: two kernels always; 1: single-pass kernel for 128 < max(Lq, Lkv) <= 256; 2: for every length <= 256
 #endif
 
+// Nothing is scheduled across a pin, and a block that holds one is not turned into selects.
+#define DMF_PIN() __builtin_amdgcn_sched_barrier(0)
+
 namespace dmf {
 
 template <int D>
@@ -160,12 +163,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
     }
     // ---- dS^T = P^T * (dP^T - delta)
     f32x16 dS;
-    const bool tail = (it + 1) * 32 > p.Lkv;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float pr = fast_exp2(S[i] - lse2);
-      if (tail && it * 32 + acc_row(i, g) >= p.Lkv) pr = 0.f;
-      dS[i] = pr * (dP[i] - delta);
+    for (int i = 0; i < 16; ++i) dS[i] = fast_exp2(S[i] - lse2) * (dP[i] - delta);
+    if ((it + 1) * 32 > p.Lkv) {   // keys past the end (last tile only); the pin keeps the selects out of the common path
+      DMF_PIN();
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (it * 32 + acc_row(i, g) >= p.Lkv) dS[i] = 0.f;
     }
     // ---- dQ^T += K^T dS^T
     {
@@ -292,7 +296,6 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     //      bounds check zero-fills them only when consecutive rows are distinct addresses, and a broadcast operand
     //      (row stride 0, e.g. the gradient of a sum over the sequence) aliases them onto row 0 instead.
     f32x16 Pm, dS;
-    const bool qtail = (it + 1) * 32 > p.Lq;   // wave-uniform
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const f32x4 l4 = *reinterpret_cast<const f32x4*>(stat + j * 8 + 4 * g);
@@ -300,11 +303,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int i = 4 * j + e;
-        float pr = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
-        if (qtail && it * 32 + acc_row(i, g) >= p.Lq) pr = 0.f;
-        Pm[i] = pr;
-        dS[i] = pr * (dP[i] - d4[e]);
+        Pm[i] = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
+        dS[i] = Pm[i] * (dP[i] - d4[e]);
       }
+    }
+    if ((it + 1) * 32 > p.Lq) {   // last tile only; the pin keeps the selects out of the common path
+      DMF_PIN();
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (it * 32 + acc_row(i, g) >= p.Lq) Pm[i] = dS[i] = 0.f;
     }
     // ---- dV^T += dout^T P ; dK^T += Q^T dS
     {
@@ -570,7 +577,6 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
       //      cycles but the issue port for 4, and a wave issues in order: only interleaved in program order do the two overlap
       //      (left alone the scheduler gathers the MFMAs, hence the pins).  Padded query rows carry lse = +inf (P = 0), padded
       //      keys are switched off where dS is handed over.
-#define DMF_PIN() __builtin_amdgcn_sched_barrier(0)
       f32x16 S = {0}, dP = {0}, Pm, dS;
       ColOperand pp[2], ds[2];
       const uint32_t xa = x_base + ((j & 3) * 8 + wave) * FC::XTILE + c32 * 64;   // this lane's key row of tile X[j % 4][wave]
