@@ -29,7 +29,14 @@ struct BwdFastCfg {
   static constexpr int STAT = 256;                    // per stage: 32 x lse, 32 x delta (fp32)
   static constexpr bool TAIL = (D % 32) != 0 && (D % 32) <= 16;   // 16-wide remainder via 16x16x32 MFMAs (72, 80)
   static constexpr int NMT = TAIL ? D / 32 : NDT;                 // full 32-wide output tiles
+  // The last 16-wide chunk of the score products has spare columns D .. (head dims 72, 104, 120).  Three of them carry
+  // a per-row constant as a bf16 triple against ones on the other side, so that the MFMA itself yields S - lse and
+  // dP - delta and the VALU subtractions go away.
+  static constexpr bool STATCOL = (D % 16) == 8;
 };
+
+// Pad vector of a tile row whose first three elements are 1.0 (see BwdFastCfg::STATCOL).
+__device__ __forceinline__ u32x4 ones3_bf16() { return u32x4{0x3f803f80u, 0x00003f80u, 0u, 0u}; }
 
 // bf16x8 chunk times a scalar, re-rounded to bf16.
 __device__ __forceinline__ u32x4 scale_bf16x8(u32x4 x, float s) {
@@ -40,13 +47,16 @@ __device__ __forceinline__ u32x4 scale_bf16x8(u32x4 x, float s) {
   return y;
 }
 
-template <int BYTES_PER_STAGE, int PADV, int P, int VPR>
+// Fills the pad vectors of a 32-row tile in both stages (the tile DMA never writes them): zeros, or with ONES the
+// 1, 1, 1, 0 ... pattern in the first pad vector.
+template <int BYTES_PER_STAGE, int PADV, int P, int VPR, bool ONES = false>
 __device__ __forceinline__ void zero_pads(char* smem, int tile_off, int tid) {
   if constexpr (PADV > 0) {
 #pragma unroll
     for (int s = 0; s < 2; ++s)
       for (int i = tid; i < 32 * PADV; i += 256)
-        *reinterpret_cast<u32x4*>(smem + s * BYTES_PER_STAGE + tile_off + ((i / PADV) * P + VPR + i % PADV) * 16) = u32x4{0, 0, 0, 0};
+        *reinterpret_cast<u32x4*>(smem + s * BYTES_PER_STAGE + tile_off + ((i / PADV) * P + VPR + i % PADV) * 16) =
+            ONES && i % PADV == 0 ? ones3_bf16() : u32x4{0, 0, 0, 0};
   }
 }
 
@@ -75,8 +85,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
 
 #pragma unroll
   for (int sub = 0; sub < SUB; ++sub) {
-    zero_pads<STAGE, P - VPR, P, VPR>(smem, sub * PAIR, tid);
-    zero_pads<STAGE, P - VPR, P, VPR>(smem, sub * PAIR + V_OFF, tid);
+    zero_pads<STAGE, P - VPR, P, VPR, F::STATCOL>(smem, sub * PAIR, tid);
+    zero_pads<STAGE, P - VPR, P, VPR, F::STATCOL>(smem, sub * PAIR + V_OFF, tid);
   }
 
   // ---- this lane's query row: Q (times scale*log2e), dout, delta, lse
@@ -101,10 +111,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
     }
   }
   const float delta = xhalf_sum(dpart);
-  float lse2 = INFINITY;   // +inf switches padded query rows off (P = 0)
+  float lse2 = 1e30f;   // switches padded query rows off (P = 0)
   if (qok) {
     lse2 = p.lse[(int64_t)bh * p.Lq + qrow] * kLog2e;
     if (g == 0) p.delta[(int64_t)bh * p.Lq + qrow] = delta;
+  }
+  if constexpr (F::STATCOL) {   // columns D .. D+2 of this row: -lse against the ones in the K tile, -delta against those in the V tile
+    if (g == 1) {
+      Qr[NCHUNK - 1] = split3_bf16(-lse2);
+      dOr[NCHUNK - 1] = split3_bf16(-delta);
+    }
   }
 
   f32x16 dQ[NMT];
@@ -164,7 +180,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
     // ---- dS^T = P^T * (dP^T - delta)
     f32x16 dS;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) dS[i] = fast_exp2(S[i] - lse2) * (dP[i] - delta);
+    for (int i = 0; i < 16; ++i) {
+      if constexpr (F::STATCOL) dS[i] = fast_exp2(S[i]) * dP[i];
+      else dS[i] = fast_exp2(S[i] - lse2) * (dP[i] - delta);
+    }
     if ((it + 1) * 32 > p.Lkv) {   // keys past the end (last tile only); the pin keeps the selects out of the common path
       DMF_PIN();
 #pragma unroll
@@ -271,79 +290,134 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     lds_barrier();
     if (it + 1 < ntiles) issue(it + 1);
-    const uint32_t ra = row_addr + (it & 1) * STAGE, ca = col_addr + (it & 1) * STAGE;
-    const float* stat = reinterpret_cast<const float*>(smem + (it & 1) * STAGE + STAT_OFF);
+    const uint32_t so = (it & 1) * STAGE;
+    const uint32_t ra = row_addr + so, ca = col_addr + so;
+    if ((it + 1) * 32 > p.Lq) {   // last tile, the whole work-group: query rows past the end get lse = +inf, i.e. P = 0 (the bounds
+      // check zero-fills their operands only when consecutive rows are distinct addresses; a broadcast operand -- row stride 0,
+      // e.g. the gradient of a sum over the sequence -- aliases them onto row 0 instead)
+      if (tid < 32 && it * 32 + tid >= p.Lq) reinterpret_cast<float*>(smem + so + STAT_OFF)[tid] = INFINITY;
+      lds_barrier();
+    }
 
-    // ---- S = Q K^T (log2 units), dP = dout V^T : rows = queries (in-lane), columns = keys (lanes)
-    f32x16 S = {0}, dP = {0};
+    // ---- Four MFMA runs per tile: S = Q K^T (log2 units) and dP = dout V^T (rows = queries, in-lane; columns = keys, lanes),
+    //      then dV^T += dout^T P and dK^T += Q^T dS.  The arithmetic in between is issued inside the run that does not depend
+    //      on it -- P = exp2(S - lse*log2e) between the MFMAs of dP, dS = P (dP - delta) between the MFMAs of dV -- because an
+    //      MFMA holds the matrix pipe for 32 cycles but the issue port for 4, and a wave issues in order: only interleaved in
+    //      program order do the two overlap (left alone the scheduler gathers the MFMAs, hence the pins).
+    //      Head dims above 96 have no registers to spare for the overlap and do the arithmetic between the runs.
+    constexpr bool IL = D <= 96;
+    f32x16 S = {0}, dP = {0}, Pm, dS;
+    ColOperand pp[2], ds[2];
+    // lse / delta of a slice's four queries (8jj + 4g .. +3): raw reads like the operands, requested one slice ahead
+    const uint32_t stat_addr = lds_addr(smem) + so + STAT_OFF + 16 * g;
+    u32x4 sl[2], sd[2];
+    auto p_slice = [&](auto jc) {
+      constexpr int jj = decltype(jc)::value;
+      const u32x4 l4 = sl[jj & 1];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) Pm[4 * jj + e] = fast_exp2(fmaf(__uint_as_float(l4[e]), -kLog2e, S[4 * jj + e]));
+      if constexpr (jj & 1) pp[jj >> 1] = acc_operand<T>(Pm, jj >> 1);
+    };
+    auto ds_slice = [&](auto jc) {
+      constexpr int jj = decltype(jc)::value;
+      const u32x4 d4 = sd[jj & 1];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dS[4 * jj + e] = Pm[4 * jj + e] * (dP[4 * jj + e] - __uint_as_float(d4[e]));
+      if constexpr (jj & 1) ds[jj >> 1] = acc_operand<T>(dS, jj >> 1);
+    };
+    static_assert(NCHUNK >= 4, "the four P slices ride between the first four dP MFMAs");
     {
       u32x4 qc[2], oc[2];
       qc[0] = lds_read128_issue<0>(ra);
-      oc[0] = lds_read128_issue<DO_OFF>(ra);
-      static_for<NCHUNK>([&](auto cc) {
+      static_for<NCHUNK>([&](auto cc) {   // run 1: S
+        constexpr int c = decltype(cc)::value;
+        if constexpr (c + 1 < NCHUNK) {
+          qc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
+          lds_read128_wait<1>(qc[c & 1]);
+        } else {   // first operand and first lse slice of the next run
+          oc[0] = lds_read128_issue<DO_OFF>(ra);
+          if constexpr (IL) sl[0] = lds_read128_issue<0>(stat_addr);
+          lds_read128_wait<IL ? 2 : 1>(qc[c & 1]);
+        }
+        mma_chunk<T>(S, qc[c & 1], Kr[c]);
+      });
+      static_for<NCHUNK>([&](auto cc) {   // run 2: dP, P formed meanwhile
         constexpr int c = decltype(cc)::value;
         constexpr bool more = c + 1 < NCHUNK;
-        if constexpr (more) {
-          qc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
-          oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
-        }
-        lds_read128_wait<more ? 2 : 0>(qc[c & 1], oc[c & 1]);
-        mma_chunk<T>(S, qc[c & 1], Kr[c]);
+        if constexpr (more) oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
+        if constexpr (IL && c + 1 < 4) sl[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(stat_addr);   // 8 queries = 32 bytes per slice
+        // operand c and lse slice c were requested one step ago: leave what has been requested since in flight
+        if constexpr (IL && c < 4) lds_read128_wait<(more ? 1 : 0) + (c + 1 < 4 ? 1 : 0)>(oc[c & 1], sl[c & 1]);
+        else lds_read128_wait<more ? 1 : 0>(oc[c & 1]);
+        DMF_PIN();
         mma_chunk<T>(dP, oc[c & 1], Vr[c]);
+        DMF_PIN();
+        if constexpr (IL && c < 4) p_slice(cc);
+        DMF_PIN();
       });
     }
-    // ---- P = exp2(S - lse*log2e), dS = P * (dP - delta).  Query rows past Lq are switched off here (P = 0): the
-    //      bounds check zero-fills them only when consecutive rows are distinct addresses, and a broadcast operand
-    //      (row stride 0, e.g. the gradient of a sum over the sequence) aliases them onto row 0 instead.
-    f32x16 Pm, dS;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(stat + j * 8 + 4 * g);
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(stat + 32 + j * 8 + 4 * g);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int i = 4 * j + e;
-        Pm[i] = fast_exp2(fmaf(l4[e], -kLog2e, S[i]));
-        dS[i] = Pm[i] * (dP[i] - d4[e]);
-      }
+    if constexpr (!IL) {   // all of the arithmetic between the runs
+      static_for<4>([&](auto jc) {
+        constexpr int jj = decltype(jc)::value;
+        sl[jj & 1] = lds_read128_issue<32 * jj>(stat_addr);
+        sd[jj & 1] = lds_read128_issue<128 + 32 * jj>(stat_addr);
+        lds_read128_wait<0>(sl[jj & 1], sd[jj & 1]);
+        p_slice(jc);
+        ds_slice(jc);
+      });
     }
-    if ((it + 1) * 32 > p.Lq) {   // last tile only; the pin keeps the selects out of the common path
-      DMF_PIN();
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (it * 32 + acc_row(i, g) >= p.Lq) Pm[i] = dS[i] = 0.f;
-    }
-    // ---- dV^T += dout^T P ; dK^T += Q^T dS
     {
-      ColOperand pp[2] = {acc_operand<T>(Pm, 0), acc_operand<T>(Pm, 1)};
-      ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
       constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
+      static_assert(NGT >= 4, "the four dS slices ride between the first four dV MFMAs");
       TrPair qq[2], oo[2];
       auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
-      qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
+      const uint32_t ta = tail_addr + so;
       oo[0] = lds_tr16_issue<lo_off(0) + DO_OFF, lo_off(0) + 8 * STR * 2 + DO_OFF>(ca);
-      static_for<NGT>([&](auto gc) {
+      if constexpr (IL) sd[0] = lds_read128_issue<128>(stat_addr);   // delta[32] follows lse[32]
+      static_for<NGT>([&](auto gc) {   // run 3: dV^T += dout^T P, dS formed meanwhile
+        constexpr int gi = decltype(gc)::value;
+        if constexpr (gi + 1 < NG) {
+          constexpr int LO = lo_off(gi + 1), HI = LO + 8 * STR * 2;
+          oo[(gi + 1) & 1] = lds_tr16_issue<LO + DO_OFF, HI + DO_OFF>(ca);
+        } else if constexpr (gi + 1 < NGT) {
+          oo[(gi + 1) & 1] = lds_tr16_issue<DO_OFF, 8 * STR * 2 + DO_OFF>(ta);
+        } else {
+          qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);   // first operand of the next run
+        }
+        if constexpr (IL && gi + 1 < 4) sd[(gi + 1) & 1] = lds_read128_issue<128 + 32 * (gi + 1)>(stat_addr);
+        if constexpr (IL && gi < 4) {
+          asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(oo[gi & 1].lo), "+v"(oo[gi & 1].hi), "+v"(sd[gi & 1]) : [n] "n"(gi + 1 < 4 ? 3 : 2));
+        } else {
+          lds_tr16_wait<2>(oo[gi & 1]);
+        }
+        DMF_PIN();
+        if constexpr (gi < NG) {
+          mma_col<T>(dV[gi % NMT], tr_operand(oo[gi & 1]), pp[gi / NMT]);
+        } else {
+          ColOperand p0, p1;
+          tail_operands(pp[0], pp[1], p0, p1);
+          mma16(dV16[0], tr_operand(oo[gi & 1]), p0);
+          mma16(dV16[1], tr_operand(oo[gi & 1]), p1);
+        }
+        DMF_PIN();
+        if constexpr (IL && gi < 4) ds_slice(gc);
+        DMF_PIN();
+      });
+      static_for<NGT>([&](auto gc) {   // run 4: dK^T += Q^T dS
         constexpr int gi = decltype(gc)::value;
         constexpr bool more = gi + 1 < NGT;
         if constexpr (gi + 1 < NG) {
           constexpr int LO = lo_off(gi + 1), HI = LO + 8 * STR * 2;
           qq[(gi + 1) & 1] = lds_tr16_issue<LO, HI>(ca);
-          oo[(gi + 1) & 1] = lds_tr16_issue<LO + DO_OFF, HI + DO_OFF>(ca);
         } else if constexpr (more) {
-          const uint32_t ta = tail_addr + (it & 1) * STAGE;
           qq[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(ta);
-          oo[(gi + 1) & 1] = lds_tr16_issue<DO_OFF, 8 * STR * 2 + DO_OFF>(ta);
         }
-        lds_tr16_wait<more ? 4 : 0>(qq[gi & 1], oo[gi & 1]);
+        lds_tr16_wait<more ? 2 : 0>(qq[gi & 1]);
         if constexpr (gi < NG) {
-          mma_col<T>(dV[gi % NMT], tr_operand(oo[gi & 1]), pp[gi / NMT]);
           mma_col<T>(dK[gi % NMT], tr_operand(qq[gi & 1]), ds[gi / NMT]);
         } else {
-          ColOperand p0, p1, d0, d1;
-          tail_operands(pp[0], pp[1], p0, p1);
+          ColOperand d0, d1;
           tail_operands(ds[0], ds[1], d0, d1);
-          mma16(dV16[0], tr_operand(oo[gi & 1]), p0);
-          mma16(dV16[1], tr_operand(oo[gi & 1]), p1);
           mma16(dK16[0], tr_operand(qq[gi & 1]), d0);
           mma16(dK16[1], tr_operand(qq[gi & 1]), d1);
         }

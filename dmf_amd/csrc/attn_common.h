@@ -74,6 +74,16 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, y);
 }
 
+// x as the sum of three bf16 numbers h + m + l (relative error 2^-24), packed into the first three elements of an
+// eight-element bf16 vector; the other five are zero.
+__device__ __forceinline__ u32x4 split3_bf16(float x) {
+  const uint32_t h = pack_bf16x2(x, 0.f);
+  const float r1 = x - __uint_as_float(h << 16);
+  const uint32_t m = pack_bf16x2(r1, 0.f);
+  const float r2 = r1 - __uint_as_float(m << 16);
+  return u32x4{h | (m << 16), pack_bf16x2(r2, 0.f), 0u, 0u};
+}
+
 // Static configuration for element type T (float or __bf16) and head dim D.
 template <typename T, int D>
 struct Cfg {
