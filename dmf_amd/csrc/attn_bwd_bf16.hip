@@ -159,60 +159,80 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
     if (it >= ntiles) break;             // wave-uniform
     const uint32_t ra = row_addr + (is & 1) * STAGE + sub * PAIR, ca = col_addr + (is & 1) * STAGE + sub * PAIR;
 
-    // ---- S^T = K Q^T (log2 units), dP^T = V dout^T
-    f32x16 S = {0}, dP = {0};
+    // ---- Three MFMA runs per 32-key tile: S^T = K Q^T (log2 units), dP^T = V dout^T, dQ^T += K^T dS^T.  P^T = exp2(S^T - lse)
+    //      is formed between the MFMAs of the dP run and the second half of dS^T = P^T (dP^T - delta) behind the first MFMA of
+    //      the dQ run (an MFMA holds the matrix pipe for 32 cycles but the issue port for 4, and a wave issues in order; left
+    //      alone the scheduler gathers the MFMAs, hence the pins).
+    f32x16 S = {0}, dP = {0}, Pm, dS;
+    ColOperand ds[2];
+    const bool tail = (it + 1) * 32 > p.Lkv;   // keys past the end (last tile only): the pin keeps the selects out of the common path
+    auto p_slice = [&](auto jc) {
+      constexpr int jj = decltype(jc)::value;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) Pm[4 * jj + e] = fast_exp2(F::STATCOL ? S[4 * jj + e] : S[4 * jj + e] - lse2);
+    };
+    auto ds_half = [&](auto hc) {
+      constexpr int hh = decltype(hc)::value;
+#pragma unroll
+      for (int i = 8 * hh; i < 8 * hh + 8; ++i) dS[i] = Pm[i] * (F::STATCOL ? dP[i] : dP[i] - delta);
+      if (tail) {
+        DMF_PIN();
+#pragma unroll
+        for (int i = 8 * hh; i < 8 * hh + 8; ++i)
+          if (it * 32 + acc_row(i, g) >= p.Lkv) dS[i] = 0.f;
+      }
+      ds[hh] = acc_operand<T>(dS, hh);
+    };
+    constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
+    TrPair kk[2];
+    auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
+    static_assert(NCHUNK >= 4, "the four P slices ride between the first four dP MFMAs");
     {
       u32x4 kc[2], vc[2];
       kc[0] = lds_read128_issue<0>(ra);
-      vc[0] = lds_read128_issue<V_OFF>(ra);
-      static_for<NCHUNK>([&](auto cc) {
+      static_for<NCHUNK>([&](auto cc) {   // run 1: S^T
         constexpr int c = decltype(cc)::value;
-        constexpr bool more = c + 1 < NCHUNK;
-        if constexpr (more) {
-          kc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
-          vc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + V_OFF>(ra);
-        }
-        lds_read128_wait<more ? 2 : 0>(kc[c & 1], vc[c & 1]);
+        if constexpr (c + 1 < NCHUNK) kc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
+        else vc[0] = lds_read128_issue<V_OFF>(ra);   // first operand of the next run
+        lds_read128_wait<1>(kc[c & 1]);
         mma_chunk<T>(S, kc[c & 1], Qr[c]);
-        mma_chunk<T>(dP, vc[c & 1], dOr[c]);
       });
-    }
-    // ---- dS^T = P^T * (dP^T - delta)
-    f32x16 dS;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if constexpr (F::STATCOL) dS[i] = fast_exp2(S[i]) * dP[i];
-      else dS[i] = fast_exp2(S[i] - lse2) * (dP[i] - delta);
-    }
-    if ((it + 1) * 32 > p.Lkv) {   // keys past the end (last tile only); the pin keeps the selects out of the common path
-      DMF_PIN();
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (it * 32 + acc_row(i, g) >= p.Lkv) dS[i] = 0.f;
-    }
-    // ---- dQ^T += K^T dS^T
-    {
-      ColOperand ds[2] = {acc_operand<T>(dS, 0), acc_operand<T>(dS, 1)};
-      constexpr int NG = 2 * NMT, NGT = NG + (TAIL ? 1 : 0);
-      TrPair kk[2];
-      auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
-      kk[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
-      static_for<NGT>([&](auto gc) {
-        constexpr int gi = decltype(gc)::value;
-        constexpr bool more = gi + 1 < NGT;
-        if constexpr (gi + 1 < NG) kk[(gi + 1) & 1] = lds_tr16_issue<lo_off(gi + 1), lo_off(gi + 1) + 8 * STR * 2>(ca);
-        else if constexpr (more) kk[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(tail_addr + (is & 1) * STAGE + sub * PAIR);
-        lds_tr16_wait<more ? 2 : 0>(kk[gi & 1]);
-        if constexpr (gi < NG) {
-          mma_col<T>(dQ[gi % NMT], tr_operand(kk[gi & 1]), ds[gi / NMT]);
-        } else {
-          ColOperand d0, d1;
-          tail_operands(ds[0], ds[1], d0, d1);
-          mma16(dQ16[0], tr_operand(kk[gi & 1]), d0);
-          mma16(dQ16[1], tr_operand(kk[gi & 1]), d1);
+      static_for<NCHUNK>([&](auto cc) {   // run 2: dP^T, P^T formed meanwhile
+        constexpr int c = decltype(cc)::value;
+        if constexpr (c + 1 < NCHUNK) {
+          vc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + V_OFF>(ra);
+          lds_read128_wait<1>(vc[c & 1]);
+        } else {   // first operand of the next run
+          kk[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);
+          lds_read128_wait<2>(vc[c & 1]);
         }
+        DMF_PIN();
+        mma_chunk<T>(dP, vc[c & 1], dOr[c]);
+        DMF_PIN();
+        if constexpr (c < 4) p_slice(cc);
+        DMF_PIN();
       });
     }
+    ds_half(std::integral_constant<int, 0>{});
+    static_for<NGT>([&](auto gc) {   // run 3: dQ^T
+      constexpr int gi = decltype(gc)::value;
+      constexpr bool more = gi + 1 < NGT;
+      if constexpr (gi + 1 < NG) kk[(gi + 1) & 1] = lds_tr16_issue<lo_off(gi + 1), lo_off(gi + 1) + 8 * STR * 2>(ca);
+      else if constexpr (more) kk[(gi + 1) & 1] = lds_tr16_issue<0, 8 * STR * 2>(tail_addr + (is & 1) * STAGE + sub * PAIR);
+      lds_tr16_wait<more ? 2 : 0>(kk[gi & 1]);
+      DMF_PIN();
+      if constexpr (gi < NG) {
+        mma_col<T>(dQ[gi % NMT], tr_operand(kk[gi & 1]), ds[gi / NMT]);
+      } else {
+        ColOperand d0, d1;
+        tail_operands(ds[0], ds[1], d0, d1);
+        mma16(dQ16[0], tr_operand(kk[gi & 1]), d0);
+        mma16(dQ16[1], tr_operand(kk[gi & 1]), d1);
+      }
+      DMF_PIN();
+      if constexpr (gi == 0) ds_half(std::integral_constant<int, 1>{});
+      DMF_PIN();
+    });
    }
   }
   store_rows_transposed<T, D, 4, NMT>(reinterpret_cast<T*>(smem), reinterpret_cast<T*>(p.dq) + base(5), p.st[5][1], q0, p.Lq, tid,
