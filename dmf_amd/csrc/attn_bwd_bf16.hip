@@ -47,17 +47,40 @@ __device__ __forceinline__ u32x4 scale_bf16x8(u32x4 x, float s) {
   return y;
 }
 
-// Fills the pad vectors of a 32-row tile in both stages (the tile DMA never writes them): zeros, or with ONES the
-// 1, 1, 1, 0 ... pattern in the first pad vector.
-template <int BYTES_PER_STAGE, int PADV, int P, int VPR, bool ONES = false>
+// Fills the pad vectors of a 32-row tile in both stages (the tile DMA never writes them) with zeros; the first pad
+// vector of a row with the 1, 1, 1, 0 ... pattern instead (PAD_ONES) or not at all (PAD_SKIP: its owner writes it).
+enum { PAD_ZERO = 0, PAD_ONES = 1, PAD_SKIP = 2 };
+template <int BYTES_PER_STAGE, int PADV, int P, int VPR, int FIRST = PAD_ZERO>
 __device__ __forceinline__ void zero_pads(char* smem, int tile_off, int tid) {
   if constexpr (PADV > 0) {
 #pragma unroll
     for (int s = 0; s < 2; ++s)
-      for (int i = tid; i < 32 * PADV; i += 256)
+      for (int i = tid; i < 32 * PADV; i += 256) {
+        if (FIRST == PAD_SKIP && i % PADV == 0) continue;
         *reinterpret_cast<u32x4*>(smem + s * BYTES_PER_STAGE + tile_off + ((i / PADV) * P + VPR + i % PADV) * 16) =
-            ONES && i % PADV == 0 ? ones3_bf16() : u32x4{0, 0, 0, 0};
+            FIRST == PAD_ONES && i % PADV == 0 ? ones3_bf16() : u32x4{0, 0, 0, 0};
+      }
   }
+}
+
+// 8-byte LDS store issued as a raw instruction, for the same reason as the untracked reads in attn_common.h (a store
+// the compiler knows about would be preceded by a full vmcnt(0) while a tile DMA is in flight).  The data is in LDS
+// once a later `s_waitcnt lgkmcnt(0)` of this wave has passed (LDS operations complete in order).
+template <int OFF>
+__device__ __forceinline__ void lds_write64_untracked(uint32_t addr, u32x2 w) {
+  asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(addr), "v"(w), "n"(OFF) : "memory");
+}
+
+template <int OFF>
+__device__ __forceinline__ void lds_write128_untracked(uint32_t addr, u32x4 w) {
+  asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(w), "n"(OFF) : "memory");
+}
+
+// 4-byte LDS read issued as a raw instruction; lgkmcnt must be waited for before the result is used.
+__device__ __forceinline__ uint32_t lds_read32_issue(uint32_t addr) {
+  uint32_t r;
+  asm volatile("ds_read_b32 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
 }
 
 // ------------------------------------------------------------------ dQ kernel
@@ -85,8 +108,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
 
 #pragma unroll
   for (int sub = 0; sub < SUB; ++sub) {
-    zero_pads<STAGE, P - VPR, P, VPR, F::STATCOL>(smem, sub * PAIR, tid);
-    zero_pads<STAGE, P - VPR, P, VPR, F::STATCOL>(smem, sub * PAIR + V_OFF, tid);
+    zero_pads<STAGE, P - VPR, P, VPR, F::STATCOL ? PAD_ONES : PAD_ZERO>(smem, sub * PAIR, tid);
+    zero_pads<STAGE, P - VPR, P, VPR, F::STATCOL ? PAD_ONES : PAD_ZERO>(smem, sub * PAIR + V_OFF, tid);
   }
 
   // ---- this lane's query row: Q (times scale*log2e), dout, delta, lse
@@ -263,8 +286,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   const int k0 = kb * 128;
   auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
 
-  zero_pads<STAGE, P - VPR, P, VPR>(smem, 0, tid);
-  zero_pads<STAGE, P - VPR, P, VPR>(smem, DO_OFF, tid);
+  // SC: column D .. D+2 of a Q row carries -lse*log2e and of a dout row -delta (bf16 triples) against ones in this lane's
+  // K and V rows, so S - lse and dP - delta come out of the MFMAs.  The stage's statistics area then holds lse / delta of
+  // the FOLLOWING tile, and one wave per tile turns them into the pad vectors of the other stage while that tile's rows
+  // are still on their way.
+  constexpr bool SC = F::STATCOL;
+  zero_pads<STAGE, P - VPR, P, VPR, SC ? PAD_SKIP : PAD_ZERO>(smem, 0, tid);
+  zero_pads<STAGE, P - VPR, P, VPR, SC ? PAD_SKIP : PAD_ZERO>(smem, DO_OFF, tid);
 
   // ---- this lane's key row: K (times scale*log2e) and V stay in registers
   u32x4 Kr[NCHUNK], Vr[NCHUNK];
@@ -275,6 +303,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     load_row_chunks<NCHUNK, VPR>(make_rows_rsrc(reinterpret_cast<const T*>(p.v) + base(3), rb_v, p.Lkv, D * 2), rb_v, krow, g, Vr);
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) Kr[c] = scale_bf16x8(Kr[c], p.scale_log2);
+    if constexpr (SC) {
+      if (g == 1) Kr[NCHUNK - 1] = Vr[NCHUNK - 1] = ones3_bf16();
+    }
   }
   f32x16 dK[NMT], dV[NMT];
   f32x4 dK16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}}, dV16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
@@ -294,11 +325,24 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     char* st = smem + (it & 1) * STAGE;
     issue_tile_rows<P, VPR>(rs_q, rb_q, (uint32_t)it * 32 * rb_q, st, wave, lane);
     issue_tile_rows<P, VPR>(rs_do, rb_do, (uint32_t)it * 32 * rb_do, st + DO_OFF, wave, lane);
-    if (wave < 2 && lane < 32)   // wave 0: lse[32], wave 1: delta[32]
+    if (wave < 2 && lane < 32)   // wave 0: lse[32], wave 1: delta[32] -- of this tile, with SC of the next one
       __builtin_amdgcn_raw_ptr_buffer_load_lds(wave == 0 ? rs_lse : rs_dl,
                                                (__attribute__((address_space(3))) void*)(st + STAT_OFF + wave * 128), 4,
-                                               lane * 4, (uint32_t)it * 128, 0, 0);
+                                               lane * 4, (uint32_t)(it + (SC ? 1 : 0)) * 128, 0, 0);
   };
+  // pad vector of row (lane % 32) of the Q tile (lanes 0..31: x = lse) or the dout tile (lanes 32..63: x = delta)
+  auto stat_vector = [&](float x, int row) {
+    if (lane < 32) return split3_bf16(row < p.Lq ? -x * kLog2e : -1e30f);   // rows past the end: P = 0
+    return split3_bf16(row < p.Lq ? -x : 0.f);
+  };
+  const uint32_t pad_addr = lds_addr(smem) + (lane < 32 ? 0 : DO_OFF) + (c32 * P + VPR) * 16;
+  if constexpr (SC) {
+    if (wave == 0) {   // tile 0
+      float x = 0.f;
+      if (c32 < p.Lq) x = (lane < 32 ? p.lse : p.delta)[(int64_t)bh * p.Lq + c32];
+      *reinterpret_cast<u32x4*>(smem + (lane < 32 ? 0 : DO_OFF) + (c32 * P + VPR) * 16) = stat_vector(x, c32);
+    }
+  }
   const uint32_t row_addr = lds_addr(smem) + c32 * STR * 2 + g * 16;
   const uint32_t col_addr = lds_addr(smem) + ((4 * g + ((lane & 15) >> 2)) * STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
@@ -312,9 +356,17 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     if (it + 1 < ntiles) issue(it + 1);
     const uint32_t so = (it & 1) * STAGE;
     const uint32_t ra = row_addr + so, ca = col_addr + so;
-    if ((it + 1) * 32 > p.Lq) {   // last tile, the whole work-group: query rows past the end get lse = +inf, i.e. P = 0 (the bounds
-      // check zero-fills their operands only when consecutive rows are distinct addresses; a broadcast operand -- row stride 0,
-      // e.g. the gradient of a sum over the sequence -- aliases them onto row 0 instead)
+    // Query rows past the end are switched off through their lse (P = 0): the bounds check zero-fills their operands only
+    // when consecutive rows are distinct addresses; a broadcast operand -- row stride 0, e.g. the gradient of a sum over
+    // the sequence -- aliases them onto row 0 instead.
+    if constexpr (SC) {
+      if (it + 1 < ntiles && wave == (it & 3)) {   // pad vectors of tile it + 1, in the other stage
+        uint32_t x = lds_read32_issue(lds_addr(smem) + so + STAT_OFF + lane * 4);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x));
+        // (in LDS before this wave's last operand read of the tile returns: LDS operations complete in order)
+        lds_write128_untracked<0>(pad_addr + (STAGE - so), stat_vector(__uint_as_float(x), (it + 1) * 32 + c32));
+      }
+    } else if ((it + 1) * 32 > p.Lq) {   // last tile, the whole work-group: lse = +inf
       if (tid < 32 && it * 32 + tid >= p.Lq) reinterpret_cast<float*>(smem + so + STAT_OFF)[tid] = INFINITY;
       lds_barrier();
     }
@@ -326,6 +378,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     //      program order do the two overlap (left alone the scheduler gathers the MFMAs, hence the pins).
     //      Head dims above 96 have no registers to spare for the overlap and do the arithmetic between the runs.
     constexpr bool IL = D <= 96;
+    constexpr bool ST = IL && !SC;   // lse / delta slices are read between the MFMAs
     f32x16 S = {0}, dP = {0}, Pm, dS;
     ColOperand pp[2], ds[2];
     // lse / delta of a slice's four queries (8jj + 4g .. +3): raw reads like the operands, requested one slice ahead
@@ -335,14 +388,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
       constexpr int jj = decltype(jc)::value;
       const u32x4 l4 = sl[jj & 1];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) Pm[4 * jj + e] = fast_exp2(fmaf(__uint_as_float(l4[e]), -kLog2e, S[4 * jj + e]));
+      for (int e = 0; e < 4; ++e) Pm[4 * jj + e] = fast_exp2(SC ? S[4 * jj + e] : fmaf(__uint_as_float(l4[e]), -kLog2e, S[4 * jj + e]));
       if constexpr (jj & 1) pp[jj >> 1] = acc_operand<T>(Pm, jj >> 1);
     };
     auto ds_slice = [&](auto jc) {
       constexpr int jj = decltype(jc)::value;
       const u32x4 d4 = sd[jj & 1];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) dS[4 * jj + e] = Pm[4 * jj + e] * (dP[4 * jj + e] - __uint_as_float(d4[e]));
+      for (int e = 0; e < 4; ++e) dS[4 * jj + e] = Pm[4 * jj + e] * (SC ? dP[4 * jj + e] : dP[4 * jj + e] - __uint_as_float(d4[e]));
       if constexpr (jj & 1) ds[jj >> 1] = acc_operand<T>(dS, jj >> 1);
     };
     static_assert(NCHUNK >= 4, "the four P slices ride between the first four dP MFMAs");
@@ -356,8 +409,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
           lds_read128_wait<1>(qc[c & 1]);
         } else {   // first operand and first lse slice of the next run
           oc[0] = lds_read128_issue<DO_OFF>(ra);
-          if constexpr (IL) sl[0] = lds_read128_issue<0>(stat_addr);
-          lds_read128_wait<IL ? 2 : 1>(qc[c & 1]);
+          if constexpr (ST) sl[0] = lds_read128_issue<0>(stat_addr);
+          lds_read128_wait<ST ? 2 : 1>(qc[c & 1]);
         }
         mma_chunk<T>(S, qc[c & 1], Kr[c]);
       });
@@ -365,9 +418,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
         constexpr int c = decltype(cc)::value;
         constexpr bool more = c + 1 < NCHUNK;
         if constexpr (more) oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
-        if constexpr (IL && c + 1 < 4) sl[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(stat_addr);   // 8 queries = 32 bytes per slice
+        if constexpr (ST && c + 1 < 4) sl[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(stat_addr);   // 8 queries = 32 bytes per slice
         // operand c and lse slice c were requested one step ago: leave what has been requested since in flight
-        if constexpr (IL && c < 4) lds_read128_wait<(more ? 1 : 0) + (c + 1 < 4 ? 1 : 0)>(oc[c & 1], sl[c & 1]);
+        if constexpr (ST && c < 4) lds_read128_wait<(more ? 1 : 0) + (c + 1 < 4 ? 1 : 0)>(oc[c & 1], sl[c & 1]);
         else lds_read128_wait<more ? 1 : 0>(oc[c & 1]);
         DMF_PIN();
         mma_chunk<T>(dP, oc[c & 1], Vr[c]);
@@ -393,7 +446,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
       auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
       const uint32_t ta = tail_addr + so;
       oo[0] = lds_tr16_issue<lo_off(0) + DO_OFF, lo_off(0) + 8 * STR * 2 + DO_OFF>(ca);
-      if constexpr (IL) sd[0] = lds_read128_issue<128>(stat_addr);   // delta[32] follows lse[32]
+      if constexpr (ST) sd[0] = lds_read128_issue<128>(stat_addr);   // delta[32] follows lse[32]
       static_for<NGT>([&](auto gc) {   // run 3: dV^T += dout^T P, dS formed meanwhile
         constexpr int gi = decltype(gc)::value;
         if constexpr (gi + 1 < NG) {
@@ -404,8 +457,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
         } else {
           qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);   // first operand of the next run
         }
-        if constexpr (IL && gi + 1 < 4) sd[(gi + 1) & 1] = lds_read128_issue<128 + 32 * (gi + 1)>(stat_addr);
-        if constexpr (IL && gi < 4) {
+        if constexpr (ST && gi + 1 < 4) sd[(gi + 1) & 1] = lds_read128_issue<128 + 32 * (gi + 1)>(stat_addr);
+        if constexpr (ST && gi < 4) {
           asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(oo[gi & 1].lo), "+v"(oo[gi & 1].hi), "+v"(sd[gi & 1]) : [n] "n"(gi + 1 < 4 ? 3 : 2));
         } else {
           lds_tr16_wait<2>(oo[gi & 1]);
@@ -455,19 +508,6 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
                                       [&](void* ws) {
                                         if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dV16[hq][e]; });
                                       });
-}
-
-// 8-byte LDS store issued as a raw instruction, for the same reason as the untracked reads in attn_common.h (a store
-// the compiler knows about would be preceded by a full vmcnt(0) while a tile DMA is in flight).  The data is in LDS
-// once a later `s_waitcnt lgkmcnt(0)` of this wave has passed (LDS operations complete in order).
-template <int OFF>
-__device__ __forceinline__ void lds_write64_untracked(uint32_t addr, u32x2 w) {
-  asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(addr), "v"(w), "n"(OFF) : "memory");
-}
-
-template <int OFF>
-__device__ __forceinline__ void lds_write128_untracked(uint32_t addr, u32x4 w) {
-  asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(w), "n"(OFF) : "memory");
 }
 
 // ------------------------------------------------ single-pass backward, whole (batch, head) unit per work-group
