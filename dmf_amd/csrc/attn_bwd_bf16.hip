@@ -11,6 +11,9 @@
 #include "attn_kernels.h"
 #include <algorithm>
 
+#ifndef DMF_DKV_WAVES
+#define DMF_DKV_WAVES 4
+#endif
 #ifndef DMF_BWD_FUSED
 #define DMF_BWD_FUSED 1   // 0: two kernels always; 1: single-pass kernel for 128 < max(Lq, Lkv) <= 256; 2: for every length <= 256
 #endif
@@ -50,12 +53,12 @@ __device__ __forceinline__ u32x4 scale_bf16x8(u32x4 x, float s) {
 // Fills the pad vectors of a 32-row tile in both stages (the tile DMA never writes them) with zeros; the first pad
 // vector of a row with the 1, 1, 1, 0 ... pattern instead (PAD_ONES) or not at all (PAD_SKIP: its owner writes it).
 enum { PAD_ZERO = 0, PAD_ONES = 1, PAD_SKIP = 2 };
-template <int BYTES_PER_STAGE, int PADV, int P, int VPR, int FIRST = PAD_ZERO>
+template <int BYTES_PER_STAGE, int PADV, int P, int VPR, int FIRST = PAD_ZERO, int NT = 256>
 __device__ __forceinline__ void zero_pads(char* smem, int tile_off, int tid) {
   if constexpr (PADV > 0) {
 #pragma unroll
     for (int s = 0; s < 2; ++s)
-      for (int i = tid; i < 32 * PADV; i += 256) {
+      for (int i = tid; i < 32 * PADV; i += NT) {
         if (FIRST == PAD_SKIP && i % PADV == 0) continue;
         *reinterpret_cast<u32x4*>(smem + s * BYTES_PER_STAGE + tile_off + ((i / PADV) * P + VPR + i % PADV) * 16) =
             FIRST == PAD_ONES && i % PADV == 0 ? ones3_bf16() : u32x4{0, 0, 0, 0};
@@ -266,8 +269,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
 }
 
 // --------------------------------------------------------------- dK/dV kernel
-template <int D>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdParams p) {
+// NW waves of 32 keys each per work-group.
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW, 8 / NW) void attn_bwd_dkv_bf16_kernel(const BwdParams p) {
   using F = BwdFastCfg<D>;
   using T = __bf16;
   constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR;
@@ -279,11 +283,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, g = lane >> 5;
-  const uint32_t nkb = (p.Lkv + 127) / 128;
+  const uint32_t nkb = (p.Lkv + 32 * NW - 1) / (32 * NW);
   const uint32_t wg = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = wg / nkb, kb = wg % nkb;
   const int b = bh / p.H, h = bh % p.H;
-  const int k0 = kb * 128;
+  const int k0 = kb * 32 * NW;
   auto base = [&](int t) { return (int64_t)b * p.st[t][0] + (int64_t)h * p.st[t][2]; };
 
   // SC: column D .. D+2 of a Q row carries -lse*log2e and of a dout row -delta (bf16 triples) against ones in this lane's
@@ -291,8 +295,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   // the FOLLOWING tile, and one wave per tile turns them into the pad vectors of the other stage while that tile's rows
   // are still on their way.
   constexpr bool SC = F::STATCOL;
-  zero_pads<STAGE, P - VPR, P, VPR, SC ? PAD_SKIP : PAD_ZERO>(smem, 0, tid);
-  zero_pads<STAGE, P - VPR, P, VPR, SC ? PAD_SKIP : PAD_ZERO>(smem, DO_OFF, tid);
+  zero_pads<STAGE, P - VPR, P, VPR, SC ? PAD_SKIP : PAD_ZERO, 64 * NW>(smem, 0, tid);
+  zero_pads<STAGE, P - VPR, P, VPR, SC ? PAD_SKIP : PAD_ZERO, 64 * NW>(smem, DO_OFF, tid);
 
   // ---- this lane's key row: K (times scale*log2e) and V stay in registers
   u32x4 Kr[NCHUNK], Vr[NCHUNK];
@@ -323,8 +327,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
   const __amdgpu_buffer_rsrc_t rs_dl = make_rows_rsrc(p.delta + (int64_t)bh * p.Lq, 4, p.Lq, 4);
   auto issue = [&](int it) {
     char* st = smem + (it & 1) * STAGE;
-    issue_tile_rows<P, VPR>(rs_q, rb_q, (uint32_t)it * 32 * rb_q, st, wave, lane);
-    issue_tile_rows<P, VPR>(rs_do, rb_do, (uint32_t)it * 32 * rb_do, st + DO_OFF, wave, lane);
+    issue_tile_rows<P, VPR, NW>(rs_q, rb_q, (uint32_t)it * 32 * rb_q, st, wave, lane);
+    issue_tile_rows<P, VPR, NW>(rs_do, rb_do, (uint32_t)it * 32 * rb_do, st + DO_OFF, wave, lane);
     if (wave < 2 && lane < 32)   // wave 0: lse[32], wave 1: delta[32] -- of this tile, with SC of the next one
       __builtin_amdgcn_raw_ptr_buffer_load_lds(wave == 0 ? rs_lse : rs_dl,
                                                (__attribute__((address_space(3))) void*)(st + STAT_OFF + wave * 128), 4,
@@ -360,7 +364,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     // when consecutive rows are distinct addresses; a broadcast operand -- row stride 0, e.g. the gradient of a sum over
     // the sequence -- aliases them onto row 0 instead.
     if constexpr (SC) {
-      if (it + 1 < ntiles && wave == (it & 3)) {   // pad vectors of tile it + 1, in the other stage
+      if (it + 1 < ntiles && wave == (it & (NW - 1))) {   // pad vectors of tile it + 1, in the other stage
         uint32_t x = lds_read32_issue(lds_addr(smem) + so + STAT_OFF + lane * 4);
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x));
         // (in LDS before this wave's last operand read of the tile returns: LDS operations complete in order)
@@ -498,12 +502,12 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_bf16_kernel(const BwdPara
     }
   }
   T* stage = reinterpret_cast<T*>(smem);
-  store_rows_transposed<T, D, 4, NMT>(stage, reinterpret_cast<T*>(p.dk) + base(6), p.st[6][1], k0, p.Lkv, tid,
+  store_rows_transposed<T, D, NW, NMT>(stage, reinterpret_cast<T*>(p.dk) + base(6), p.st[6][1], k0, p.Lkv, tid,
                                       [&](int t, int i) { return dK[t][i] * p.scale; },
                                       [&](void* ws) {
                                         if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dK16[hq][e] * p.scale; });
                                       });
-  store_rows_transposed<T, D, 4, NMT>(stage, reinterpret_cast<T*>(p.dv) + base(7), p.st[7][1], k0, p.Lkv, tid,
+  store_rows_transposed<T, D, NW, NMT>(stage, reinterpret_cast<T*>(p.dv) + base(7), p.st[7][1], k0, p.Lkv, tid,
                                       [&](int t, int i) { return dV[t][i]; },
                                       [&](void* ws) {
                                         if constexpr (TAIL) store_tail16<T, D, NMT>(ws, lane, [&](int hq, int e) { return dV16[hq][e]; });
@@ -997,17 +1001,19 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
   using F = BwdFastCfg<D>;
   constexpr int tiles = 2 * (2 * F::TBYTES + F::STAT) + 512;
   constexpr int stage = 128 * Cfg<__bf16, D>::OROWV * 16;
-  constexpr int smem = tiles > stage ? tiles : stage;
+  constexpr int kKvWaves = DMF_DKV_WAVES;
+  constexpr int stage2 = 32 * kKvWaves * Cfg<__bf16, D>::OROWV * 16;
+  constexpr int smem = tiles > stage2 ? tiles : stage2;
   constexpr int kDqSub = 2;   // two 32-key tiles per barrier in the dQ kernel (+3 % over one; four would leave one work-group per CU)
   constexpr int tiles1 = 2 * kDqSub * 2 * F::TBYTES + 512;
   constexpr int smem1 = tiles1 > stage ? tiles1 : stage;
   auto k1 = attn_bwd_dq_bf16_kernel<D, kDqSub>;
-  auto k2 = attn_bwd_dkv_bf16_kernel<D>;
+  auto k2 = attn_bwd_dkv_bf16_kernel<D, kKvWaves>;
   static bool lds_ok1[64] = {}, lds_ok2[64] = {};
   if (!ensure_dynamic_lds(k1, smem1, lds_ok1) || !ensure_dynamic_lds(k2, smem, lds_ok2)) return -7;
-  const uint32_t nqb = (p.Lq + 127) / 128, nkb = (p.Lkv + 127) / 128;
+  const uint32_t nqb = (p.Lq + 127) / 128, nkb = (p.Lkv + 32 * kKvWaves - 1) / (32 * kKvWaves);
   if (int rc = launch_kernel(k1, dim3(nqb * (uint32_t)BH), dim3(256), smem1, stream, p)) return rc;
-  return launch_kernel(k2, dim3(nkb * (uint32_t)BH), dim3(256), smem, stream, p);
+  return launch_kernel(k2, dim3(nkb * (uint32_t)BH), dim3(64 * kKvWaves), smem, stream, p);
 }
 
 // Returns 1 if there is no tuned kernel for the case (caller uses the generic ones).

@@ -124,6 +124,7 @@ def test_reference_family(l, h, d):
 # ---- edge cases: ragged and tiny sequences, cross-attention lengths --------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("Lq,Lkv", [(1, 1), (16, 16), (64, 64), (100, 77), (129, 65), (257, 300), (128, 33),
+                                    (520, 300), (290, 1000),
                                     (160, 200), (256, 130), (130, 256), (255, 40), (224, 256)])   # (the last five: single-pass backward)
 def test_ragged_lengths(Lq, Lkv, dtype):
     _parity(2, Lq, 2, 72, dtype, seed=Lq * 7 + Lkv, Lkv=Lkv)
@@ -216,7 +217,7 @@ def test_full_size_properties(B, L):
     _check("lse fused vs primal-only", lse, lse2.float().cpu(), 1e-6)
 
 
-@pytest.mark.parametrize("Lq,Lkv", [(77, 77), (100, 130)])
+@pytest.mark.parametrize("Lq,Lkv", [(77, 77), (100, 130), (300, 290)])
 def test_backward_with_broadcast_gradient(Lq, Lkv):
     """The gradient of ``o.sum(1)`` reaches the backward as an expanded tensor whose
     sequence stride is 0: every query row, including the rows a partial last tile
