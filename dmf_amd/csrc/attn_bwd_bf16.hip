@@ -23,10 +23,22 @@
 
 namespace dmf {
 
-template <int D>
+// Tile row pitch in 16-byte vectors.  Odd, so that the row-operand reads (ds_read_b128, 16 lanes a cycle over 64 banks)
+// are conflict-free; with TRFREE also such that four consecutive rows start at least two vectors apart modulo 16, so
+// that a transposed read (ds_read_b64_tr_b16: 16 lanes fetch 32 bytes of each of four consecutive rows) is
+// conflict-free too -- pitches of 11 or 17 vectors put rows 0 and 3 (0 and 1) on the same banks and cost the read a
+// second cycle.
+constexpr int bwd_tile_pitch(int min_vectors, bool trfree) {
+  for (int p = min_vectors | 1;; p += 2) {
+    const int m = p % 16;
+    if (!trfree || m == 3 || m == 7 || m == 9 || m == 13) return p;
+  }
+}
+
+template <int D, bool TRFREE = false>
 struct BwdFastCfg {
   static constexpr int VPR = D / 8, NCHUNK = (D + 15) / 16, NDT = (D + 31) / 32;
-  static constexpr int P = Cfg<__bf16, D>::ROWV;     // tile row pitch in 16-byte vectors (odd): tiles are read both by rows and transposed
+  static constexpr int P = TRFREE ? bwd_tile_pitch(Cfg<__bf16, D>::ROWV0, true) : Cfg<__bf16, D>::ROWV;   // tiles are read both by rows and transposed
   static constexpr int STR = P * 8;
   static constexpr int TBYTES = 32 * P * 16;          // one 32-row tile
   static constexpr int STAT = 256;                    // per stage: 32 x lse, 32 x delta (fp32)
@@ -90,7 +102,7 @@ __device__ __forceinline__ uint32_t lds_read32_issue(uint32_t addr) {
 // SUB = 32-key tiles per stage (and per work-group barrier).
 template <int D, int SUB>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParams p) {
-  using F = BwdFastCfg<D>;
+  using F = BwdFastCfg<D, true>;
   using T = __bf16;
   constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR;
   constexpr bool TAIL = F::TAIL;
@@ -272,7 +284,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_bf16_kernel(const BwdParam
 // NW waves of 32 keys each per work-group.
 template <int D, int NW>
 __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_bwd_dkv_bf16_kernel(const BwdParams p) {
-  using F = BwdFastCfg<D>;
+  using F = BwdFastCfg<D, true>;
   using T = __bf16;
   constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR;
   constexpr bool TAIL = F::TAIL;
@@ -998,7 +1010,7 @@ static int launch_bwd_fused_t(const BwdParams& p, int BH, hipStream_t stream) {
 
 template <int D>
 static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
-  using F = BwdFastCfg<D>;
+  using F = BwdFastCfg<D, true>;
   constexpr int tiles = 2 * (2 * F::TBYTES + F::STAT) + 512;
   constexpr int stage = 128 * Cfg<__bf16, D>::OROWV * 16;
   constexpr int kKvWaves = DMF_DKV_WAVES;
