@@ -130,6 +130,13 @@ def test_ragged_lengths(Lq, Lkv, dtype):
     _parity(2, Lq, 2, 72, dtype, seed=Lq * 7 + Lkv, Lkv=Lkv)
 
 
+@pytest.mark.parametrize("L", [200, 300, 1024])
+def test_peaked_softmax_inputs(L):
+    """Inputs of twice the contract's scale: logits up to +-30, |lse| up to 25 -- the range in which the statistics folded
+    into spare head-dim columns (backward, D = 72) would show a lossy encoding; both backward schemes (single pass at 200)."""
+    _parity(2, L, 2, 72, torch.bfloat16, seed=5, std=2.0)
+
+
 def test_packed_qkv_strided_views_match_contiguous():
     """q, k, v (and tangents) as views into a packed (B, L, 3, H, D) buffer with
     strides (3LHD, 3HD, D, 1), the layout models/layers.py:143-147 produces."""
