@@ -534,8 +534,26 @@ static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
   return launch_fast_q<D, JVP, NW, false, false>(p, BH, stream);
 }
 
-// Work-group width policy: 256-row work-groups (one per CU, half the tile traffic per FLOP) when the sequence fills them.
-static bool fwd_wide_workgroups(int Lq) { return Lq > 128; }
+// Work-group width policy.  256-row work-groups (8 waves, one per CU with tangents) fetch every key tile once per 256
+// queries -- half the tile traffic per FLOP -- and are the default when the sequence fills them.  128-row work-groups
+// are resident two per CU (three where the kernel needs at most 168 registers: head dim 64 with tangents), so one's
+// first and last rows overlap another's tiles.  Measured on MI355X (fwd+JVP, 8 waves vs 4):
+//   * head dim 64, three per CU: 4 waves win once the grid gives every CU three of them
+//     (B64 N1024 0.779 -> 0.749 ms, B256 N256 0.293 -> 0.269, B64 H12 N256 0.056 -> 0.048; smaller grids lose);
+//   * other head dims, N <= 256: 4 waves win only where 8-wave work-groups would run in two or three rounds
+//     (B32 H16: 0.0438 -> 0.0413 ms, B48: 0.070 -> 0.062) and lose 2-3 % from four rounds on;
+//   * without tangents the 8-wave kernel already fits twice per CU and is never slower.
+static bool fwd_wide_workgroups(int Lq, int D, bool jvp, int BH) {
+  if (Lq <= 128) return false;
+  if (!jvp) return true;
+  const int cus = compute_units();
+  if (D == 64) return (int64_t)BH * ((Lq + 127) / 128) < 3 * (int64_t)cus;
+  if (Lq <= 256) {
+    const int64_t rounds = ((int64_t)BH * ((Lq + 255) / 256) + cus - 1) / cus;
+    return rounds < 2 || rounds > 3;
+  }
+  return true;
+}
 
 // Returns 1 if this translation unit has no kernel for the case (caller falls
 // back to the generic kernel), else 0 / negative error code.
@@ -544,7 +562,7 @@ int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_
   int64_t max_row = std::max(std::max(p.st[0][1], p.st[1][1]), p.st[2][1]);
   if (jvp) max_row = std::max(max_row, std::max(std::max(p.st[3][1], p.st[4][1]), p.st[5][1]));
   if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 256) >= (int64_t)1 << 31) return 1;
-  const bool wide = fwd_wide_workgroups(p.Lq);
+  const bool wide = fwd_wide_workgroups(p.Lq, D, jvp, BH);
 #define DMF_CASE(DD)                                                                           \
   case DD:                                                                                     \
     if (wide) return jvp ? launch_fast_t<DD, true, 8>(p, BH, stream) : launch_fast_t<DD, false, 8>(p, BH, stream); \

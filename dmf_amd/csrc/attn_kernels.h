@@ -54,6 +54,18 @@ inline bool ensure_dynamic_lds(K kernel, int bytes, bool (&done)[64]) {
 }
 
 
+// Compute units of the current device (asked once per device; 256 if the query fails).
+inline int compute_units() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    cached[dev] = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
+  }
+  return cached[dev];
+}
+
 // Launch `kernel(params)` and return 0 or -7 (DMF_ATTN_ELAUNCH).  The status is the one hipLaunchKernel returns for
 // this launch; the process-wide "last error" is neither read nor cleared, so an error left behind by somebody
 // else's earlier call is not reported as a failure of this library (nor hidden from its owner).
