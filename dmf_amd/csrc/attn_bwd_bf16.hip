@@ -1,12 +1,14 @@
-// Tuned bf16 backward (dQ kernel + dK/dV kernel) for gfx950.
+// Tuned bf16 backward for gfx950: the dQ kernel + dK/dV kernel pair (any length) and the single-pass kernel for
+// sequences of at most 256 rows (further down).
 //
-// Same two-kernel, atomics-free scheme and the same register layouts as the
-// generic kernels in attn_bwd.hip, with the throughput structure of the tuned
-// forward: <= 256 VGPRs (two work-groups per CU), 32-row tiles streamed
-// HBM -> LDS by bounds-checked buffer DMA into a double buffer with one barrier
-// per tile, software-pipelined LDS operand reads, and the softmax scale and
-// log2(e) folded into the register-resident operand (Q in the dQ kernel, K in
-// the dK/dV kernel) so that P = exp2(S - lse*log2e) costs one VALU op + exp.
+// The pair is the two-kernel, atomics-free scheme of the generic kernels in attn_bwd.hip with the same register
+// layouts and the throughput structure of the tuned forward: 32-row tiles streamed HBM -> LDS by bounds-checked
+// buffer DMA into a double buffer with one barrier per tile, software-pipelined LDS operand reads, the softmax scale
+// and log2(e) folded into the register-resident operand (Q in the dQ kernel, K in the dK/dV kernel).  Per tile each
+// kernel issues its products as separate MFMA runs with the P / dS arithmetic pinned between the MFMAs of the run that
+// does not depend on it; the end-of-sequence selects sit behind wave-uniform branches (last tile only); at head dim 72
+// the statistics (-lse*log2e, -delta) ride in spare head-dim columns so that S - lse and dP - delta come out of the
+// MFMAs (BwdFastCfg::STATCOL); tile pitches are free of bank conflicts for row and transposed reads alike.
 #include "attn_common.h"
 #include "attn_kernels.h"
 #include <algorithm>
