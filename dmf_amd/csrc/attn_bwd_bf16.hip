@@ -1037,7 +1037,11 @@ int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream) 
   if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 256) >= (int64_t)1 << 31) return 1;
   // whole (batch, head) units per work-group, every score tile formed once
   const int Lmax = std::max(p.Lq, p.Lkv);
-  if (Lmax <= 256 && (DMF_BWD_FUSED == 2 || (DMF_BWD_FUSED == 1 && Lmax > 128))) {
+  // (head dim 64: the two kernels need 124 / 166 registers and are resident four / three work-groups per CU; from one
+  //  (batch, head) unit per CU on they are as fast as the single pass or faster -- B32 H12 N256 0.048 -> 0.042 ms,
+  //  B128 0.161 -> 0.150, B256 H16 equal -- and only a grid smaller than the device loses, 0.025 -> 0.029 at B16 H12)
+  const bool pair_wins = D == 64 && BH >= compute_units();
+  if (Lmax <= 256 && !pair_wins && (DMF_BWD_FUSED == 2 || (DMF_BWD_FUSED == 1 && Lmax > 128))) {
     switch (D) {
       case 64: return launch_bwd_fused_t<64>(p, BH, stream);
       case 72: return launch_bwd_fused_t<72>(p, BH, stream);
