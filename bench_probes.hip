@@ -45,15 +45,35 @@ __global__ __launch_bounds__(256) void mfma_loop(float* out, int iters, int rand
 }
 
 typedef __attribute__((ext_vector_type(4))) uint32_t vec16;
+// One work-group per (batch, head); consecutive heads of a batch element are placed on one XCD (the hardware deals
+// work-group ids round robin over the 8 XCDs), so that the cache lines two adjacent 144-byte head rows share are
+// fetched into one L2 -- without that the strided pattern streams at 3.7-3.9 TB/s instead of 4.6 -- and every thread
+// keeps four rows' worth of loads in flight.
+constexpr int kStreamUnroll = 4;
 __global__ __launch_bounds__(256) void rows_stream(const vec16* __restrict__ a0, const vec16* __restrict__ a1, const vec16* __restrict__ a2,
                                                    const vec16* __restrict__ a3, const vec16* __restrict__ a4, const vec16* __restrict__ a5,
                                                    vec16* __restrict__ o0, vec16* __restrict__ o1, int H, int N, int vpr, int head_contiguous) {
-  const int bh = blockIdx.x, b = bh / H, h = bh % H;
-  for (int v = threadIdx.x; v < N * vpr; v += 256) {
-    const int n = v / vpr, cv = v % vpr;
-    const size_t idx = head_contiguous ? (((size_t)b * H + h) * N + n) * vpr + cv : (((size_t)b * N + n) * H + h) * vpr + cv;
-    o0[idx] = a0[idx] ^ a1[idx] ^ a2[idx];
-    o1[idx] = a3[idx] ^ a4[idx] ^ a5[idx];
+  const uint32_t total_wgs = gridDim.x;
+  const int bh = total_wgs % 8 == 0 ? (blockIdx.x % 8) * (total_wgs / 8) + blockIdx.x / 8 : blockIdx.x;
+  const int b = bh / H, h = bh % H, total = N * vpr;
+  for (int v0 = threadIdx.x; v0 < total; v0 += 256 * kStreamUnroll) {
+    vec16 x[kStreamUnroll][6];
+    size_t idx[kStreamUnroll];
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u) {
+      const int v = v0 + u * 256, n = v / vpr, cv = v % vpr;
+      idx[u] = head_contiguous ? (((size_t)b * H + h) * N + n) * vpr + cv : (((size_t)b * N + n) * H + h) * vpr + cv;
+      if (v < total) {
+        x[u][0] = a0[idx[u]]; x[u][1] = a1[idx[u]]; x[u][2] = a2[idx[u]];
+        x[u][3] = a3[idx[u]]; x[u][4] = a4[idx[u]]; x[u][5] = a5[idx[u]];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u)
+      if (v0 + u * 256 < total) {
+        o0[idx[u]] = x[u][0] ^ x[u][1] ^ x[u][2];
+        o1[idx[u]] = x[u][3] ^ x[u][4] ^ x[u][5];
+      }
   }
 }
 
