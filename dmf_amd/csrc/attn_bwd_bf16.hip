@@ -579,11 +579,17 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
   float* stat_lse = reinterpret_cast<float*>(smem + FC::STAT_OFF);
   float* stat_delta = stat_lse + 256;
 
-  // ---- zero the contraction padding of the K tiles and of both Q / dout stages
+  // SC: columns D .. D+2 of a Q row carry -lse*log2e and of a dout row -delta (bf16 triples, BwdFastCfg::STATCOL) against
+  // ones in this lane's K and V rows, so that S - lse and dP - delta come out of the MFMAs; the lane that finishes a
+  // row's delta writes both pad vectors.
+  constexpr bool SC = F::STATCOL;
+  // ---- zero the contraction padding of the K tiles and of both Q / dout stages (with SC not the first pad vector of
+  //      the stage tiles: its owner writes it, for tile 0 before the first barrier)
   if constexpr (P > VPR) {
     constexpr int PADV = P - VPR;
     for (int i = tid; i < (8 + 2 * NST) * 32 * PADV; i += 512) {
       const int tile = i / (32 * PADV), r = (i / PADV) % 32, cv = VPR + i % PADV;
+      if (SC && tile >= 8 && cv == VPR) continue;
       *reinterpret_cast<u32x4*>(smem + tile * TB + (r * P + cv) * 16) = u32x4{0, 0, 0, 0};
     }
   }
@@ -622,10 +628,14 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
   // vector of dout and of o per lane (lanes past the head dim read zeros), summed across the 16 lanes.
   const uint32_t rb_o = (uint32_t)p.st[4][1] * 2;
   const __amdgpu_buffer_rsrc_t rs_o = make_rows_rsrc(reinterpret_cast<const T*>(p.o) + base(4), rb_o, p.Lq, D * 2);
-  struct DeltaRows { u32x4 d, o; };
+  struct DeltaRows { u32x4 d, o; float lse; };
   auto delta_request = [&](int j) {
     const int qrow = 32 * j + (tid >> 4), cv = tid & 15;
     DeltaRows r;
+    r.lse = 0.f;
+    if constexpr (SC) {
+      if (cv == 15 && qrow < p.Lq) r.lse = p.lse[(int64_t)bh * p.Lq + qrow];
+    }
     r.d = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_do, cv < VPR ? (uint32_t)qrow * rb_do + cv * 16 : 0x7ffffff0u, 0, 0));
     r.o = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_o, cv < VPR ? (uint32_t)qrow * rb_o + cv * 16 : 0x7ffffff0u, 0, 0));
     return r;
@@ -648,12 +658,20 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
     const int qrow = 32 * j + (tid >> 4);
     if ((tid & 15) == 15) {
       const bool qok = qrow < p.Lq;
-      stat_delta[qrow] = qok ? s : 0.f;
+      if constexpr (SC) {   // rows past the end: P = 0 through a huge "lse"
+        char* row = smem + FC::QS_OFF + (j % NST) * STAGE + ((tid >> 4) * P + VPR) * 16;
+        *reinterpret_cast<u32x4*>(row) = split3_bf16(qok ? -r.lse * kLog2e : -1e30f);
+        *reinterpret_cast<u32x4*>(row + DO_OFF) = split3_bf16(qok ? -s : 0.f);
+      } else {
+        stat_delta[qrow] = qok ? s : 0.f;
+      }
       if (qok) p.delta[(int64_t)bh * p.Lq + qrow] = s;
     }
   };
 
-  if (tid < 256) stat_lse[tid] = tid < p.Lq ? p.lse[(int64_t)bh * p.Lq + tid] : INFINITY;   // +inf switches padded query rows off (P = 0)
+  if constexpr (!SC) {
+    if (tid < 256) stat_lse[tid] = tid < p.Lq ? p.lse[(int64_t)bh * p.Lq + tid] : INFINITY;   // +inf switches padded query rows off (P = 0)
+  }
   DeltaRows dr = delta_request(0);
   issue_q(0);
   // ---- this wave's 32 key rows, whole rows by DMA: K straight into its tile of the LDS-resident copy (the phase 2
@@ -679,7 +697,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
 #pragma unroll
     for (int c = 0; c + 1 < NCHUNK; ++c) asm volatile("" : "+v"(Vr[c]));
     if constexpr (2 * NCHUNK > VPR) {
-      if (g == 1) Vr[NCHUNK - 1] = u32x4{0, 0, 0, 0};
+      if (g == 1) Vr[NCHUNK - 1] = SC ? ones3_bf16() : u32x4{0, 0, 0, 0};
     }
   }
   delta_finish(0, dr);
@@ -712,6 +730,9 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
     for (int c = 0; c + 1 < NCHUNK; ++c) asm volatile("" : "+v"(Kr[c]));
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) Kr[c] = scale_bf16x8(Kr[c], p.scale_log2);
+    if constexpr (SC) {
+      if (g == 1) Kr[NCHUNK - 1] = ones3_bf16();
+    }
     for (int j = 4 * half; j < j_end; ++j) {
       if (j == 0 || j != 4 * half) {   // (the first tile of a later half was waited for before the dQ rows were stored)
         wait_tile(j);     // this wave's share of tile j has landed
@@ -734,20 +755,22 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
       const uint32_t xa = x_base + ((j & 3) * 8 + wave) * FC::XTILE + c32 * 64;   // this lane's key row of tile X[j % 4][wave]
       // lse / delta of the slice's four queries: raw reads like the operands, requested one slice ahead (a tracked read
       // would be waited for with lgkmcnt(0), i.e. together with the operand reads just issued behind it)
+      //      (With SC both statistics are already inside S and dP and none of this is read.)
+      constexpr bool ST = !SC;
       const uint32_t stat_addr = lds_addr(stat_lse) + (j * 32 + 4 * g) * 4;
       u32x4 sl[2], sd[2];
       auto p_slice = [&](auto jc) {   // elements 4jj .. 4jj+3: queries 8jj + 4g .. +3 of the tile
         constexpr int jj = decltype(jc)::value;
         const u32x4 l4 = sl[jj & 1];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) Pm[4 * jj + e] = fast_exp2(fmaf(__uint_as_float(l4[e]), -kLog2e, S[4 * jj + e]));
+        for (int e = 0; e < 4; ++e) Pm[4 * jj + e] = fast_exp2(SC ? S[4 * jj + e] : fmaf(__uint_as_float(l4[e]), -kLog2e, S[4 * jj + e]));
         if constexpr (jj & 1) pp[jj >> 1] = acc_operand<T>(Pm, jj >> 1);
       };
       auto ds_slice = [&](auto jc) {
         constexpr int jj = decltype(jc)::value;
         const u32x4 d4 = sd[jj & 1];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dS[4 * jj + e] = Pm[4 * jj + e] * (dP[4 * jj + e] - __uint_as_float(d4[e]));
+        for (int e = 0; e < 4; ++e) dS[4 * jj + e] = Pm[4 * jj + e] * (SC ? dP[4 * jj + e] : dP[4 * jj + e] - __uint_as_float(d4[e]));
         if constexpr (jj & 1) {
           ds[jj >> 1] = acc_operand<T>(dS, jj >> 1);
           // dS tile -> X (zeros for keys past the end: their K rows must not reach dQ)
@@ -760,27 +783,24 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
       };
       static_assert(NCHUNK >= 4, "the four P slices ride between the first four dP MFMAs");
       {
-        u32x4 qc[2], oc[2];
-        qc[0] = lds_read128_issue<0>(ra);
-        static_for<NCHUNK>([&](auto cc) {   // run 1: S
+        // run 1: S.  All of its operands are requested at once (a wave alone on its SIMD would otherwise wait out one LDS
+        // latency per MFMA), then the first operand and the first lse slice of the next run.
+        u32x4 qc[NCHUNK], oc[2];
+        static_for<NCHUNK>([&](auto cc) { qc[decltype(cc)::value] = lds_read128_issue<32 * decltype(cc)::value>(ra); });
+        oc[0] = lds_read128_issue<DO_OFF>(ra);
+        if constexpr (ST) sl[0] = lds_read128_issue<0>(stat_addr);
+        static_for<NCHUNK>([&](auto cc) {
           constexpr int c = decltype(cc)::value;
-          if constexpr (c + 1 < NCHUNK) {
-            qc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ra);
-            lds_read128_wait<1>(qc[c & 1]);
-          } else {   // first operand and first lse slice of the next run
-            oc[0] = lds_read128_issue<DO_OFF>(ra);
-            sl[0] = lds_read128_issue<0>(stat_addr);
-            lds_read128_wait<2>(qc[c & 1]);
-          }
-          mma_chunk<T>(S, qc[c & 1], Kr[c]);
+          lds_read128_wait<NCHUNK - 1 - c + (ST ? 2 : 1)>(qc[c]);
+          mma_chunk<T>(S, qc[c], Kr[c]);
         });
         static_for<NCHUNK>([&](auto cc) {   // run 2: dP, P formed meanwhile
           constexpr int c = decltype(cc)::value;
           constexpr bool more = c + 1 < NCHUNK;
           if constexpr (more) oc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DO_OFF>(ra);
-          if constexpr (c + 1 < 4) sl[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(stat_addr);   // 8 queries = 32 bytes per slice
+          if constexpr (ST && c + 1 < 4) sl[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(stat_addr);   // 8 queries = 32 bytes per slice
           // operand c and lse slice c were requested one step ago: leave what has been requested since in flight
-          if constexpr (c < 4) lds_read128_wait<(more ? 1 : 0) + (c + 1 < 4 ? 1 : 0)>(oc[c & 1], sl[c & 1]);
+          if constexpr (ST && c < 4) lds_read128_wait<(more ? 1 : 0) + (c + 1 < 4 ? 1 : 0)>(oc[c & 1], sl[c & 1]);
           else lds_read128_wait<more ? 1 : 0>(oc[c & 1]);
           DMF_PIN();
           mma_chunk<T>(dP, oc[c & 1], Vr[c]);
@@ -796,7 +816,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
         auto lo_off = [](int gi) constexpr { return (16 * (gi / NMT) * STR + 32 * (gi % NMT)) * 2; };
         const uint32_t ta = lds_addr(smem) + tail_off + stage_off;
         oo[0] = lds_tr16_issue<lo_off(0) + DO_OFF, lo_off(0) + 8 * STR * 2 + DO_OFF>(ca);
-        sd[0] = lds_read128_issue<1024>(stat_addr);   // stat_delta = stat_lse + 256 floats
+        if constexpr (ST) sd[0] = lds_read128_issue<1024>(stat_addr);   // stat_delta = stat_lse + 256 floats
         static_for<NGT>([&](auto gc) {   // run 3: dV^T += dout^T P, dS formed and handed over meanwhile
           constexpr int gi = decltype(gc)::value;
           if constexpr (gi + 1 < NG) {
@@ -807,8 +827,8 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
           } else {
             qq[0] = lds_tr16_issue<lo_off(0), lo_off(0) + 8 * STR * 2>(ca);   // first operand of the next run
           }
-          if constexpr (gi + 1 < 4) sd[(gi + 1) & 1] = lds_read128_issue<1024 + 32 * (gi + 1)>(stat_addr);
-          if constexpr (gi < 4) {
+          if constexpr (ST && gi + 1 < 4) sd[(gi + 1) & 1] = lds_read128_issue<1024 + 32 * (gi + 1)>(stat_addr);
+          if constexpr (ST && gi < 4) {
             asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(oo[gi & 1].lo), "+v"(oo[gi & 1].hi), "+v"(sd[gi & 1]) : [n] "n"(gi + 1 < 4 ? 3 : 2));
           } else {
             lds_tr16_wait<2>(oo[gi & 1]);
