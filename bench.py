@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # summaries in profiles/attn_<kernel>_bf16_d72_<workload>.txt).  The two-kernel backward at N=1024 reads q, k, v, dout twice.
 MEASURED_TRAFFIC_BYTES = {("fwd_jvp", "xl2_512px"): 1.2124e9, ("fwd_jvp", "xl2_256px"): 1.2123e9,
                           ("fwd", "xl2_512px"): 6.0844e8, ("fwd", "xl2_256px"): 6.0936e8,
-                          ("bwd", "xl2_512px"): 1.8712e9, ("bwd", "xl2_256px"): 1.2838e9}
+                          ("bwd", "xl2_512px"): 1.8712e9, ("bwd", "xl2_256px"): 1.2502e9}
 
 DEVICE_WAKE_SECONDS = 0.3        # untimed launches of the measured kernel before the --warmup steps (clock ramp from idle)
 
@@ -166,7 +166,7 @@ PROFILE_FILES = {("fwd_jvp", "xl2_512px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_5
 # Share of the clocked cycles in which the MFMA pipe was busy (SQ_VALU_MFMA_BUSY_CYCLES / (4 SQ_BUSY_CU_CYCLES)), from the
 # rocprofv3 --pmc runs summarised in the files above (offline, like `traffic`); None where no such run is committed.
 MEASURED_MFMA_BUSY = {("fwd_jvp", "xl2_512px"): 0.585, ("fwd_jvp", "xl2_256px"): 0.354, ("fwd", "xl2_512px"): 0.491,
-                      ("fwd", "xl2_256px"): 0.277, ("bwd", "xl2_512px"): 0.515, ("bwd", "xl2_256px"): 0.193}
+                      ("fwd", "xl2_256px"): 0.277, ("bwd", "xl2_512px"): 0.515, ("bwd", "xl2_256px"): 0.195}
 
 
 def roofline(name, ms, kind="fwd_jvp"):
