@@ -82,6 +82,29 @@ def test_xl2_shape_reduced_batch(L, dtype):
     _parity(2 if L == 256 else 1, L, 16, 72, dtype, seed=3 if L == 256 else 4)
 
 
+@pytest.mark.parametrize("B,H,D", [(32, 16, 72), (64, 12, 64)])
+def test_model_call_shapes_take_the_narrow_work_groups(B, H, D):
+    """The attention calls of DMFT-XL/2 at batch 32 and DMFT-B/2 at batch 64 (N = 256): grids for which the forward
+    launcher picks 128-row work-groups with tangents (two or three rounds of 256-row ones, resp. head dim 64) and, at
+    head dim 64, the backward launcher the kernel pair.  Sampled (batch, head) units against the oracle, and the
+    fused forward against the primal-only one, which keeps 256-row work-groups."""
+    L, dtype, scale = 256, torch.bfloat16, D ** -0.5
+    g = torch.Generator(device=DEV).manual_seed(B + D)
+    q, k, v, tq, tk, tv, do = (torch.randn(B, L, H, D, generator=g, device=DEV).to(dtype) for _ in range(7))
+    o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)[:3]
+    o2, lse2 = _lib.fwd(q, k, v, scale)
+    dq, dk, dv = _lib.bwd(do, q, k, v, o2, lse2, scale)
+    _check("o fused vs primal-only", o, o2.float().cpu(), 1e-3)
+    _check("lse fused vs primal-only", lse, lse2.float().cpu(), 1e-6)
+    for b, h in ((0, 0), (B // 2, H // 2), (B - 1, H - 1)):
+        sl = lambda t: t[b:b + 1, :, h:h + 1].float().cpu()
+        o_ref, to_ref = ao.base_attn_jvp(*(sl(t) for t in (q, k, v, tq, tk, tv)))
+        _check(f"o[{b},{h}]", sl(o), o_ref, 2e-2)
+        _check(f"to[{b},{h}]", sl(to), to_ref, 2e-2)
+        for name, got, exp in zip(("dq", "dk", "dv"), (dq, dk, dv), ao.base_attn_grads(*(sl(t) for t in (q, k, v, do)))):
+            _check(f"{name}[{b},{h}]", sl(got), exp, 2e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("D", [32, 64, 72, 80, 96, 128])
 def test_all_head_dims(D, dtype):
