@@ -32,12 +32,38 @@ if ROOT not in sys.path:
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per step of each entry point, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over
-# `bench.py --workload W --kernel K` (each scaled by what the counter reads for a plain 1 GiB copy in the same run;
-# summaries in profiles/attn_<kernel>_bf16_d72_<workload>.txt).  The two-kernel backward at N=1024 reads q, k, v, dout twice.
-MEASURED_TRAFFIC_BYTES = {("fwd_jvp", "xl2_512px"): 1.2124e9, ("fwd_jvp", "xl2_256px"): 1.2123e9,
-                          ("fwd", "xl2_512px"): 6.0844e8, ("fwd", "xl2_256px"): 6.0936e8,
-                          ("bwd", "xl2_512px"): 1.8712e9, ("bwd", "xl2_256px"): 1.2502e9}
+# Counter figures measured offline with rocprofv3 --pmc over `bench.py --workload W --kernel K` (summaries with the
+# commands in profiles/attn_<kernel>_bf16_d72_<workload>.txt): HBM bytes per step from FETCH_SIZE / WRITE_SIZE, each scaled
+# by what the counter reads for a plain 1 GiB copy in the same run, and the share of the clocked cycles in which the MFMA
+# pipe was busy (SQ_VALU_MFMA_BUSY_CYCLES / (4 SQ_BUSY_CU_CYCLES)).  Each row names the kernel it was taken on and the
+# hash of that kernel's source files at the time (source_hash()); a row whose kernel or hash no longer matches what
+# this tree launches is reported as stale and its figures are withheld.  The two-kernel backward at N=1024 reads
+# q, k, v, dout twice.
+OFFLINE_COUNTERS = {
+    ("fwd_jvp", "xl2_512px"): {"traffic": 1.2124e9, "mfma_busy": 0.585, "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>",
+                               "src": ("attn_fwd_bf16.hip", "4122c577d5636135")},
+    ("fwd_jvp", "xl2_256px"): {"traffic": 1.2123e9, "mfma_busy": 0.354, "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>",
+                               "src": ("attn_fwd_bf16.hip", "4122c577d5636135")},
+    ("fwd", "xl2_512px"): {"traffic": 6.0844e8, "mfma_busy": 0.491, "kernel": "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>",
+                           "src": ("attn_fwd_bf16.hip", "4122c577d5636135")},
+    ("fwd", "xl2_256px"): {"traffic": 6.0936e8, "mfma_busy": 0.277, "kernel": "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>",
+                           "src": ("attn_fwd_bf16.hip", "4122c577d5636135")},
+    ("bwd", "xl2_512px"): {"traffic": 1.8712e9, "mfma_busy": 0.515,
+                           "kernel": "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72, 4>", "src": ("attn_bwd_bf16.hip", "307092ee0438a48c")},
+    ("bwd", "xl2_256px"): {"traffic": 1.2502e9, "mfma_busy": 0.195, "kernel": "dmf::attn_bwd_fused_bf16_kernel<72>",
+                           "src": ("attn_bwd_bf16.hip", "307092ee0438a48c")},
+}
+
+
+def source_hash(name):
+    """First 16 hex digits of the SHA-256 of a kernel source file together with the shared device header."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in (name, "attn_common.h"):
+        with open(os.path.join(ROOT, "dmf_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
 
 DEVICE_WAKE_SECONDS = 0.3        # untimed launches of the measured kernel before the --warmup steps (clock ramp from idle)
 
@@ -156,28 +182,22 @@ def cpu_baseline_config1():
     return out
 
 
-# Kernels behind each entry point at the two workloads (rocprofv3 names), and where the offline counter figures live.
-KERNELS = {"fwd_jvp": "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>", "fwd": "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>",
-           "bwd": {"xl2_512px": "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72, 4>",
-                   "xl2_256px": "dmf::attn_bwd_fused_bf16_kernel<72>"}}
-PROFILE_FILES = {("fwd_jvp", "xl2_512px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_512px.txt", ("fwd_jvp", "xl2_256px"): "profiles/attn_fwd_jvp_bf16_d72_xl2_256px.txt",
-                 ("fwd", "xl2_512px"): "profiles/attn_fwd_bf16_d72_xl2_512px.txt", ("fwd", "xl2_256px"): "profiles/attn_fwd_bf16_d72_xl2_256px.txt",
-                 ("bwd", "xl2_512px"): "profiles/attn_bwd_bf16_d72_xl2_512px.txt", ("bwd", "xl2_256px"): "profiles/attn_bwd_bf16_d72_xl2_256px.txt"}
-# Share of the clocked cycles in which the MFMA pipe was busy (SQ_VALU_MFMA_BUSY_CYCLES / (4 SQ_BUSY_CU_CYCLES)), from the
-# rocprofv3 --pmc runs summarised in the files above (offline, like `traffic`); None where no such run is committed.
-MEASURED_MFMA_BUSY = {("fwd_jvp", "xl2_512px"): 0.585, ("fwd_jvp", "xl2_256px"): 0.354, ("fwd", "xl2_512px"): 0.491,
-                      ("fwd", "xl2_256px"): 0.277, ("bwd", "xl2_512px"): 0.515, ("bwd", "xl2_256px"): 0.195}
+PROFILE_FILES = {(k, w): f"profiles/attn_{k}_bf16_d72_{w}.txt" for k in ("fwd_jvp", "fwd", "bwd") for w in ("xl2_512px", "xl2_256px")}
 
 
 def roofline(name, ms, kind="fwd_jvp"):
     """Roofline entry for one kernel-level measurement: the MFMA roof when the workload's arithmetic intensity is above
     the machine balance (2.5 PFLOP/s / 8 TB/s = 312 FLOP/B), the HBM roof otherwise (fwd+JVP at N=256: 191 FLOP/B)."""
+    from dmf_amd import _lib
     B, H, N, D, _ = WORKLOADS[name]
     flops, nbytes = attn_flops(B, H, N, D, kind), attn_bytes(B, H, N, D, kind)
-    kern = KERNELS[kind]
-    common = {"traffic": MEASURED_TRAFFIC_BYTES.get((kind, name)),
-              "traffic_source": PROFILE_FILES[(kind, name)] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, offline)",
-              "mfma_busy": MEASURED_MFMA_BUSY.get((kind, name)), "kernel": kern if isinstance(kern, str) else kern[name]}
+    kernel = _lib.plan(kind, B, H, N, N, D)       # what the library launches for this shape on this device
+    off = OFFLINE_COUNTERS.get((kind, name))
+    fresh = off is not None and off["kernel"] == kernel and off["src"][1] == source_hash(off["src"][0])
+    common = {"traffic": off["traffic"] if fresh else None,
+              "traffic_source": (PROFILE_FILES[(kind, name)] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, offline)") if fresh
+                                else "withheld: the committed counter run was taken on another kernel or kernel source",
+              "mfma_busy": off["mfma_busy"] if fresh else None, "kernel": kernel}
     if flops / nbytes >= MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
         a = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": a / MFMA_BF16_PEAK_TFLOPS,
@@ -306,15 +326,15 @@ class _Telemetry:
         return out
 
 
-def power_probes(fns):
-    """Board power, shader clock and the SMU's throttler residencies while each of the named GPU workloads runs for two
-    seconds (None without sysfs access)."""
+def power_probes(fns, seconds=2.0):
+    """Board power, shader clock and the SMU's throttler residencies while each of the named GPU workloads runs for
+    ``seconds`` (None without sysfs access)."""
     tel = _Telemetry()
     if not tel.available():
         return None
     out = {"power_cap_w": tel.cap_w}
     for label, fn in fns:
-        out[label] = tel.measure(fn)
+        out[label] = tel.measure(fn, seconds=seconds)
     probe = os.path.join(ROOT, "libbench_probes.so")
     if os.path.exists(probe):   # the register-only MFMA loop of device_probes(): what pure matrix work draws (each call is synchronous)
         import ctypes
@@ -323,7 +343,7 @@ def power_probes(fns):
         lib.dmf_probe_mfma_tflops.argtypes = [ctypes.c_int, ctypes.c_int]
         for label, rnd in (("mfma_loop_random_operands", 1), ("mfma_loop_constant_operands", 0)):
             rates = []
-            out[label] = tel.measure(lambda: rates.append(lib.dmf_probe_mfma_tflops(rnd, 20000)), burst=1)
+            out[label] = tel.measure(lambda: rates.append(lib.dmf_probe_mfma_tflops(rnd, 20000)), seconds=seconds, burst=1)
             if out[label] is not None and rates:
                 out[label]["tflops_mean"] = sum(rates) / len(rates)
     return out
@@ -397,6 +417,9 @@ def main():
                          "train_dmf.py:427, with the new value 'hip')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
+    ap.add_argument("--all-cases", action="store_true",
+                    help="also run the end-to-end cases outside the two BASELINE model configurations (no-grad forward, 512px training "
+                         "step, whole DMF loss step, SiT flow-matching step, sampling loop) and every variant of each case")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch one plain 1 GiB device copy (reads 1 GiB, writes 1 GiB): the known-size kernel "
                          "that HBM traffic counters are scaled by when this command runs under rocprofv3 --pmc")
@@ -476,6 +499,7 @@ def main():
 
     if not args.no_extra:
         extra = {}
+        rows = []
         o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)
         for wname in WORKLOADS:
             Bw, Hw, Nw, Dw, _ = WORKLOADS[wname]
@@ -491,43 +515,74 @@ def main():
                              ("bwd", lambda: _lib.bwd(dow, qw, kw, vw, ow, lsew, scale))):
                 t_ms, _ = time_gpu(fn, max(10, args.steps // 2), max(5, args.warmup // 2))
                 fl, by = attn_flops(Bw, Hw, Nw, Dw, kind), attn_bytes(Bw, Hw, Nw, Dw, kind)
+                rl = roofline(wname, t_ms, kind)
                 row[kind] = {"ms": t_ms, "tflops": fl / t_ms / 1e9, "pct_bf16_mfma_peak": 100 * fl / t_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS,
                              "hbm_gbs_algorithmic": by / t_ms / 1e6, "pct_hbm_peak": 100 * by / t_ms / 1e6 / HBM_PEAK_GBS,
-                             "roofline": roofline(wname, t_ms, kind)}
+                             "roofline": rl}
+                rows.append({"workload": f"{wname} B{Bw} H{Hw} N{Nw} D{Dw}", "entry": kind, "kernel": rl["kernel"], "ms": round(t_ms, 4),
+                             "bound": rl["bound"], "frac": round(rl["frac"], 4), "tflops": round(fl / t_ms / 1e9, 1),
+                             "hbm_gbs": round(by / t_ms / 1e6, 1),
+                             "traffic_ratio": None if rl["traffic"] is None else round(rl["traffic"] / by, 3),
+                             "mfma_busy": rl["mfma_busy"]})
             extra[wname] = row
             progress(f"{wname}: fwd_jvp / fwd / bwd = " + " / ".join(f"{row[kd]['ms']:.4f}" for kd in ("fwd_jvp", "fwd", "bwd")) + " ms")
             del ins
+        # every kernel-level figure of the path in one compact list (the bulky detail stays under "extra")
+        result["roofline_rows"] = rows
         extra["device_probes"] = device_probes()
-        zq = torch.zeros_like(q)
+        zq = [torch.zeros_like(q) for _ in range(6)]
         other = "xl2_256px" if name == "xl2_512px" else "xl2_512px"
         q2, k2, v2, tq2, tk2, tv2, do2 = make_inputs(other, dev, dtype, seed=3)
         o2, _, lse2 = _lib.fwd_jvp(q2, k2, v2, tq2, tk2, tv2, scale)
-        zq2 = torch.zeros_like(q2)
+        zq2 = [torch.zeros_like(q2) for _ in range(6)]
+        # (all-zero inputs: six separate tensors, so that the memory footprint -- and with it what the caches hold --
+        #  is that of the real call and only the operand toggling differs)
         extra["power"] = power_probes([
             (f"attn_fwd_jvp_{name}", lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)),
-            (f"attn_fwd_jvp_{name}_all_zero_inputs", lambda: _lib.fwd_jvp(zq, zq, zq, zq, zq, zq, scale)),
+            (f"attn_fwd_jvp_{name}_all_zero_inputs", lambda: _lib.fwd_jvp(*zq, scale)),
             (f"attn_bwd_{name}", lambda: _lib.bwd(do, q, k, v, o, lse, scale)),
             (f"attn_fwd_jvp_{other}", lambda: _lib.fwd_jvp(q2, k2, v2, tq2, tk2, tv2, scale)),
-            (f"attn_fwd_jvp_{other}_all_zero_inputs", lambda: _lib.fwd_jvp(zq2, zq2, zq2, zq2, zq2, zq2, scale)),
+            (f"attn_fwd_jvp_{other}_all_zero_inputs", lambda: _lib.fwd_jvp(*zq2, scale)),
             (f"attn_bwd_{other}", lambda: _lib.bwd(do2, q2, k2, v2, o2, lse2, scale)),
-        ])
+        ] if args.all_cases else [
+            (f"attn_fwd_jvp_{name}", lambda: _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)),
+            (f"attn_fwd_jvp_{name}_all_zero_inputs", lambda: _lib.fwd_jvp(*zq, scale)),
+        ], seconds=2.0 if args.all_cases else 1.0)
+        if extra["power"] is not None:
+            pw = extra["power"].get(f"attn_fwd_jvp_{name}") or {}
+            result["power"] = {"cap_w": extra["power"].get("power_cap_w"), "fwd_jvp_w_mean": pw.get("power_w_mean"),
+                               "fwd_jvp_sclk_mhz_mean": pw.get("sclk_mhz_mean"),
+                               "fwd_jvp_ppt_residency_pct": (pw.get("throttler_residency_pct") or {}).get("ppt_pwr")}
         del zq, zq2, q2, k2, v2, tq2, tk2, tv2, do2, o2, lse2
         progress("device probes done" + ("" if extra["power"] is None else f"; power {json.dumps(extra['power'])}"))
-        extra["block_kernels"] = block_kernel_rows(dev)
-        progress("block kernels done")
+        if args.all_cases:
+            extra["block_kernels"] = block_kernel_rows(dev)
+            progress("block kernels done")
         try:
             from dmf_amd import harness
-            extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10), log=progress)
+            # default: the two model configurations BASELINE names (DMFT-B/2 forward+JVP at batch 64, DMFT-XL/2 training step at
+            # batch 32) and the caller of the headline attention shape, fused graph replay against the naive operator
+            only = None if args.all_cases else ("DMFT-B/2", "DMFT-XL/2", "DMFT-XL/2 512px qk-norm")
+            variants = None if args.all_cases else ("hip_fused_graph", "hip", "base")
+            extra["dmft"] = harness.bench_dmft(steps=max(3, args.steps // 10), log=progress, only=only, variants=variants)
+            result["images_per_s"] = {
+                key: {v: round(extra["dmft"][key][f"{v}_images_per_s"], 1) for v in ("hip_fused_graph", "hip", "base")
+                      if f"{v}_images_per_s" in extra["dmft"][key]}
+                for key in ("DMFT-B/2", "DMFT-XL/2", "DMFT-XL/2 512px qk-norm") if key in extra["dmft"]}
+            result["images_per_s"]["cases"] = {"DMFT-B/2": "forward+JVP, batch 64, 256px, bf16 autocast (BASELINE config 2)",
+                                               "DMFT-XL/2": "forward+JVP+backward, batch 32, 256px, bf16 autocast (BASELINE config 5)",
+                                               "DMFT-XL/2 512px qk-norm": "forward+JVP, batch 16, 1024 tokens, qk-norm (caller of the headline shape)"}
         except ImportError:
             pass
-        result["extra"] = extra
 
     if not args.no_cpu:
         progress("CPU baseline (bounded sample) ...")
         result["cpu_baseline"] = cpu_baseline(name)
         if not args.no_extra:
-            result["extra"]["cpu_config1"] = cpu_baseline_config1()
+            result["cpu_config1"] = cpu_baseline_config1()
 
+    if not args.no_extra:
+        result["extra"] = extra     # last: the bulky detail behind the compact keys above
     print(json.dumps(result))
 
 

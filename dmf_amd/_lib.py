@@ -38,6 +38,7 @@ SIGNATURES = {
     "dmf_attn_fwd_qnorm": (c_int, [_P] * 7 + [_F] + [_P] * 4 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_fwd_qknorm": (c_int, [_P] * 8 + [_F] + [_P] * 6 + [_S] + [_I] * 5 + [_F, _I, _P]),
     "dmf_attn_bwd": (c_int, [_P] * 10 + [_S] + [_I] * 5 + [_F, _I, _P]),
+    "dmf_attn_plan": (c_int, [_I] * 7 + [ctypes.c_char_p, _I]),
     "dmf_block_workspace_floats": (c_int64, [_I] * 4),
     "dmf_ln_modulate_fwd": (c_int, [_P] * 8 + [_S] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
     "dmf_ln_modulate_bwd": (c_int, [_P] * 8 + [_L] + [_I] * 3 + [_F] + [_I] * 3 + [_P]),
@@ -77,6 +78,18 @@ def load() -> ctypes.CDLL:
 def _check(rc: int, what: str) -> None:
     if rc != 0:
         raise RuntimeError(f"{what} failed: {load().dmf_attn_strerror(rc).decode()} (code {rc})")
+
+
+PLAN_ENTRIES = {"fwd": 0, "fwd_jvp": 1, "bwd": 2, "fwd_qnorm_jvp": 3, "fwd_qknorm_jvp": 4}
+
+
+def plan(entry: str, B: int, H: int, Lq: int, Lkv: int, D: int, dtype=torch.bfloat16) -> str:
+    """Name(s) of the kernel(s) the entry point ``entry`` launches for this shape on the current
+    device, as profilers print them (``dmf_attn_plan``; host-only, launches nothing)."""
+    buf = ctypes.create_string_buffer(256)
+    code = DMF_ATTN_BF16 if dtype == torch.bfloat16 else DMF_ATTN_F32
+    _check(load().dmf_attn_plan(PLAN_ENTRIES[entry], B, H, Lq, Lkv, D, code, buf, len(buf)), "dmf_attn_plan")
+    return buf.value.decode()
 
 
 def _dtype_code(t: torch.Tensor) -> int:

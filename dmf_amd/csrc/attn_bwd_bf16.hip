@@ -12,18 +12,21 @@
 #include "attn_common.h"
 #include "attn_kernels.h"
 #include <algorithm>
-
-#ifndef DMF_DKV_WAVES
-#define DMF_DKV_WAVES 4
-#endif
-#ifndef DMF_BWD_FUSED
-#define DMF_BWD_FUSED 1   // 0: two kernels always; 1: single-pass kernel for 128 < max(Lq, Lkv) <= 256; 2: for every length <= 256
-#endif
+#include <cstdio>
 
 // Nothing is scheduled across a pin, and a block that holds one is not turned into selects.
 #define DMF_PIN() __builtin_amdgcn_sched_barrier(0)
 
 namespace dmf {
+
+// Waves per dK/dV work-group: four (eight halve the L2 -> LDS tile traffic but measured equal at head dim 72 and 8 % slower
+// at head dim 64, where they leave one work-group per CU instead of three).
+constexpr int kKvWaves = 4;
+// 32-key tiles per barrier in the dQ kernel: two (+3 % over one; four would leave one work-group per CU).
+constexpr int kDqSub = 2;
+// The single-pass kernel takes sequences of 129 .. 256 rows; up to 128 rows a (batch, head) unit would occupy half of
+// its eight waves and the kernel pair is faster.
+constexpr int kFusedMinRows = 129, kFusedMaxRows = 256;
 
 // Tile row pitch in 16-byte vectors.  Odd, so that the row-operand reads (ds_read_b128, 16 lanes a cycle over 64 banks)
 // are conflict-free; with TRFREE also such that four consecutive rows start at least two vectors apart modulo 16, so
@@ -1035,10 +1038,8 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
   using F = BwdFastCfg<D, true>;
   constexpr int tiles = 2 * (2 * F::TBYTES + F::STAT) + 512;
   constexpr int stage = 128 * Cfg<__bf16, D>::OROWV * 16;
-  constexpr int kKvWaves = DMF_DKV_WAVES;
   constexpr int stage2 = 32 * kKvWaves * Cfg<__bf16, D>::OROWV * 16;
   constexpr int smem = tiles > stage2 ? tiles : stage2;
-  constexpr int kDqSub = 2;   // two 32-key tiles per barrier in the dQ kernel (+3 % over one; four would leave one work-group per CU)
   constexpr int tiles1 = 2 * kDqSub * 2 * F::TBYTES + 512;
   constexpr int smem1 = tiles1 > stage ? tiles1 : stage;
   auto k1 = attn_bwd_dq_bf16_kernel<D, kDqSub>;
@@ -1050,24 +1051,37 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
   return launch_kernel(k2, dim3(nkb * (uint32_t)BH), dim3(64 * kKvWaves), smem, stream, p);
 }
 
+// Policy: does the single-pass kernel take this case?  Whole (batch, head) units per work-group, every score tile formed
+// once.  (Head dim 64: the two kernels need 124 / 166 registers and are resident four / three work-groups per CU; from one
+// (batch, head) unit per CU on they are as fast as the single pass or faster -- B32 H12 N256 0.048 -> 0.042 ms,
+// B128 0.161 -> 0.150, B256 H16 equal -- and only a grid smaller than the device loses, 0.025 -> 0.029 at B16 H12.
+// Head dim 128: K, the tile stages and the exchange area exceed the LDS.)
+bool bwd_single_pass(int Lq, int Lkv, int D, int BH) {
+  const int Lmax = std::max(Lq, Lkv);
+  if (D != 64 && D != 72 && D != 80 && D != 96) return false;
+  if (D == 64 && BH >= compute_units()) return false;
+  return Lmax >= kFusedMinRows && Lmax <= kFusedMaxRows;
+}
+
+bool plan_bwd_bf16_fast(int Lq, int Lkv, int D, int BH, char* buf, size_t n) {
+  if (D != 64 && D != 72 && D != 80 && D != 96 && D != 128) return false;
+  if (bwd_single_pass(Lq, Lkv, D, BH)) snprintf(buf, n, "dmf::attn_bwd_fused_bf16_kernel<%d>", D);
+  else snprintf(buf, n, "dmf::attn_bwd_dq_bf16_kernel<%d, %d> + dmf::attn_bwd_dkv_bf16_kernel<%d, %d>", D, kDqSub, D, kKvWaves);
+  return true;
+}
+
 // Returns 1 if there is no tuned kernel for the case (caller uses the generic ones).
 int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream) {
   // 32-bit buffer addressing: every (batch, head) slab of rows must span < 2 GiB
   const int64_t max_row = std::max(std::max(std::max(p.st[0][1], p.st[1][1]), std::max(p.st[2][1], p.st[3][1])), p.st[4][1]);
   if (max_row * 2 * (int64_t)(std::max(p.Lq, p.Lkv) + 256) >= (int64_t)1 << 31) return 1;
-  // whole (batch, head) units per work-group, every score tile formed once
-  const int Lmax = std::max(p.Lq, p.Lkv);
-  // (head dim 64: the two kernels need 124 / 166 registers and are resident four / three work-groups per CU; from one
-  //  (batch, head) unit per CU on they are as fast as the single pass or faster -- B32 H12 N256 0.048 -> 0.042 ms,
-  //  B128 0.161 -> 0.150, B256 H16 equal -- and only a grid smaller than the device loses, 0.025 -> 0.029 at B16 H12)
-  const bool pair_wins = D == 64 && BH >= compute_units();
-  if (Lmax <= 256 && !pair_wins && (DMF_BWD_FUSED == 2 || (DMF_BWD_FUSED == 1 && Lmax > 128))) {
+  if (bwd_single_pass(p.Lq, p.Lkv, D, BH)) {
     switch (D) {
       case 64: return launch_bwd_fused_t<64>(p, BH, stream);
       case 72: return launch_bwd_fused_t<72>(p, BH, stream);
       case 80: return launch_bwd_fused_t<80>(p, BH, stream);
       case 96: return launch_bwd_fused_t<96>(p, BH, stream);
-      default: break;   // head dim 128: K, the tile stages and the exchange area exceed the LDS
+      default: break;
     }
   }
   switch (D) {

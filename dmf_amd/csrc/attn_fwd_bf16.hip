@@ -24,6 +24,7 @@
 #include "attn_common.h"
 #include "attn_kernels.h"
 #include <algorithm>
+#include <cstdio>
 
 namespace dmf {
 
@@ -306,7 +307,8 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
           ss = fmaf(x[e], x[e], ss);
           if constexpr (JVP) st = fmaf(x[e], t[e], st);
         }
-        const float r = 1.f / sqrtf(group16_sum(ss) * (1.f / D) + p.q_eps);
+        // (rows past the end of the sequence were zero-filled and must stay zero: with eps == 0 their r would be infinite)
+        const float r = it * BKV + row < p.Lkv ? 1.f / sqrtf(group16_sum(ss) * (1.f / D) + p.q_eps) : 0.f;
         const float dr = JVP ? -r * r * r * group16_sum(st) * (1.f / D) : 0.f;
         if (live) {
           u32x4 kn, tkn;
@@ -552,6 +554,14 @@ static bool fwd_wide_workgroups(int Lq, int D, bool jvp, int BH) {
     const int64_t rounds = ((int64_t)BH * ((Lq + 255) / 256) + cus - 1) / cus;
     return rounds < 2 || rounds > 3;
   }
+  return true;
+}
+
+bool plan_fwd_bf16_fast(int Lq, int D, bool jvp, int BH, bool q_norm, bool k_norm, char* buf, size_t n) {
+  if (D != 64 && D != 72 && D != 80 && D != 96 && D != 128) return false;
+  const auto tf = [](bool x) { return x ? "true" : "false"; };
+  snprintf(buf, n, "dmf::attn_fwd_bf16_kernel<%d, %s, %d, %s, %s>", D, tf(jvp), fwd_wide_workgroups(Lq, D, jvp, BH) ? 8 : 4,
+           tf(q_norm), tf(q_norm && k_norm));
   return true;
 }
 

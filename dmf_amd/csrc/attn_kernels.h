@@ -67,12 +67,16 @@ inline int compute_units() {
 }
 
 // Launch `kernel(params)` and return 0 or -7 (DMF_ATTN_ELAUNCH).  The status is the one hipLaunchKernel returns for
-// this launch; the process-wide "last error" is neither read nor cleared, so an error left behind by somebody
-// else's earlier call is not reported as a failure of this library (nor hidden from its owner).
+// this launch.  An error left behind by somebody else's earlier call is neither reported as a failure of this library
+// nor hidden from its owner: the process-wide "last error" is only read -- and thereby cleared -- when this very launch
+// failed, so that the failure the caller already gets as a return code is not raised a second time by the next
+// unrelated check of the runtime's error state.
 template <typename P>
 inline int launch_kernel(void (*kernel)(P), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, P params) {
   void* args[] = {&params};
-  return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, args, lds_bytes, stream) == hipSuccess ? 0 : -7;
+  if (hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, args, lds_bytes, stream) == hipSuccess) return 0;
+  (void)hipGetLastError();
+  return -7;
 }
 
 // Return 0 or a negative DMF_ATTN_E* code.
@@ -84,5 +88,11 @@ int launch_fwd_bf16_fast(const FwdParams& p, int BH, int D, bool jvp, hipStream_
 int launch_bwd_generic(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream);
 int launch_bwd_bf16_fast(const BwdParams& p, int BH, int D, hipStream_t stream);
 int launch_bwd(const BwdParams& p, int BH, int D, bool bf16, hipStream_t stream);
+
+// Host-only: the tuned kernel(s) the two *_bf16_fast launchers pick for a case, written to buf as profilers spell them
+// ("dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>", the backward pair joined by " + "), for rows less than
+// 2 GiB apart.  Returns false when there is no tuned kernel (the generic ones run).
+bool plan_fwd_bf16_fast(int Lq, int D, bool jvp, int BH, bool q_norm, bool k_norm, char* buf, size_t n);
+bool plan_bwd_bf16_fast(int Lq, int Lkv, int D, int BH, char* buf, size_t n);
 
 }  // namespace dmf

@@ -3,6 +3,8 @@
 // allocates, frees or synchronises.
 #include "../../include/dmf_attn.h"
 #include "attn_kernels.h"
+#include <algorithm>
+#include <cstdio>
 
 namespace {
 
@@ -121,6 +123,26 @@ int dmf_attn_fwd_jvp(const void* q, const void* k, const void* v, const void* tq
 int dmf_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int64_t* strides,
                  int B, int H, int Lq, int Lkv, int D, float scale, int dtype, void* stream) {
   return fwd_impl(q, k, v, nullptr, nullptr, nullptr, o, nullptr, lse, nullptr, strides, false, B, H, Lq, Lkv, D, scale, dtype, stream);
+}
+
+int dmf_attn_plan(int entry, int B, int H, int Lq, int Lkv, int D, int dtype, char* buf, int buflen) {
+  if (int rc = check_common(B, H, Lq, Lkv, D, dtype)) return rc;
+  if (buf == nullptr || buflen < 1) return DMF_ATTN_ENULL;
+  if (entry < DMF_ATTN_PLAN_FWD || entry > DMF_ATTN_PLAN_FWD_QKNORM_JVP) return DMF_ATTN_ESHAPE;
+  const bool bf16 = dtype == DMF_ATTN_BF16;
+  const char* t = bf16 ? "__bf16" : "float";
+  const size_t n = (size_t)buflen;
+  if (entry == DMF_ATTN_PLAN_BWD) {
+    if (!(bf16 && dmf::plan_bwd_bf16_fast(Lq, Lkv, D, B * H, buf, n)))
+      snprintf(buf, n, "dmf::attn_bwd_dq_kernel<%s, %d> + dmf::attn_bwd_dkv_kernel<%s, %d>", t, D, t, D);
+    return DMF_ATTN_OK;
+  }
+  const bool jvp = entry == DMF_ATTN_PLAN_FWD_JVP || entry == DMF_ATTN_PLAN_FWD_QNORM_JVP || entry == DMF_ATTN_PLAN_FWD_QKNORM_JVP;
+  const bool qn = entry >= DMF_ATTN_PLAN_FWD_QNORM_JVP, kn = entry == DMF_ATTN_PLAN_FWD_QKNORM_JVP;
+  if (bf16 && dmf::plan_fwd_bf16_fast(Lq, D, jvp, B * H, qn, kn, buf, n)) return DMF_ATTN_OK;
+  if (qn) return DMF_ATTN_ENOKERNEL;
+  snprintf(buf, n, "dmf::attn_fwd_kernel<%s, %d, %s>", t, D, jvp ? "true" : "false");
+  return DMF_ATTN_OK;
 }
 
 int dmf_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* o, const float* lse,

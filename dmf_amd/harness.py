@@ -215,12 +215,17 @@ def build_model(name: str, attn_func: str, device, qk_norm: bool = False, input_
 def stale_grad_accumulator(p: torch.Tensor) -> bool:
     """True if an autograd graph that is still alive refers to ``p``'s gradient accumulator.  The accumulator node is
     created on first use and freed with the last graph that points at it; asking for it twice returns the same
-    object only while something else keeps it alive."""
+    object only while something else keeps it alive.  Anything else that legitimately holds the accumulator --
+    a post-accumulate-grad hook, a DDP-style reducer -- reads as "stale" too.  Works under ``torch.no_grad()``
+    (the probe switches gradient mode on for itself); a tensor that does not require a gradient has no accumulator."""
+    if not p.requires_grad:
+        return False
     key = "dmf_amd.stale_probe"
-    node = p.view_as(p).grad_fn.next_functions[0][0]
-    node.metadata[key] = True          # lives on the node itself, not on this Python wrapper
-    del node
-    node = p.view_as(p).grad_fn.next_functions[0][0]
+    with torch.enable_grad():
+        node = p.view_as(p).grad_fn.next_functions[0][0]
+        node.metadata[key] = True          # lives on the node itself, not on this Python wrapper
+        del node
+        node = p.view_as(p).grad_fn.next_functions[0][0]
     alive = bool(node.metadata.pop(key, False))
     return alive
 
@@ -301,7 +306,7 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
     ``hip_fused``       -- the same, launched eagerly through ``torch.func.jvp`` (the reference's call),
     ``hip``             -- 'hip' attention inside the reference's tensor expressions,
     ``base``            -- naive attention (the reference's own CPU-runnable operator).
-    ``only`` / ``variants`` restrict the model / the variants that are run; ``log(text)``
+    ``only`` (a key or a collection of keys) / ``variants`` restrict the cases / the variants that are run; ``log(text)``
     is called after every measurement."""
     out = {}
     # (key, model, batch, dmf_depth, mode, latent size, qk_norm)
@@ -312,7 +317,8 @@ def bench_dmft(steps: int = 5, device="cuda:0", compare_base: bool = True, only=
                  ("DMFT-XL/2 DMF loss step (mg)", "DMFT-XL/2", 16, 20, "dmf_loss", 32, False),
                  ("SiT-XL/2 FM train step", "SiT-XL/2", 32, None, "fm", 32, False),
                  ("DMFT-XL/2 4-step sampling cfg 1.5", "DMFT-XL/2", 64, 20, "sample", 32, False)]
-    cases = [c for c in all_cases if only in (None, c[0])]
+    wanted = None if only is None else ({only} if isinstance(only, str) else set(only))
+    cases = [c for c in all_cases if wanted is None or c[0] in wanted]
     all_variants = [("hip_fused_graph", "hip", "hip", True), ("hip_fused_fwad", "hip", "hip", False), ("hip_fused", "hip", "hip", False),
                     ("hip", "hip", "torch", False)]
     if compare_base:

@@ -163,6 +163,29 @@ DMF_ATTN_API int dmf_attn_bwd(const void* dout, const void* q, const void* k, co
                  int B, int H, int Lq, int Lkv, int D,
                  float scale, int dtype, void* stream);
 
+/*
+ * Host-only query: which kernel(s) a call of an entry point would launch for a
+ * shape on the current device, written to `buf` (NUL-terminated, truncated to
+ * buflen) in the spelling profilers print, e.g.
+ * "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>"; the two kernels of
+ * the backward pair are joined by " + ".  Launches nothing and reads no device
+ * memory; the answer depends on the device's compute-unit count (work-group
+ * width and single-pass-vs-pair policies) and assumes rows less than 2 GiB
+ * apart.  No counterpart in the reference (its dispatch is the Python branch
+ * at models/flash_attention_2_jvp.py:190-191); meant for tests and benchmarks
+ * that must name the kernel they exercised.  DMF_ATTN_ENOKERNEL for a
+ * q-norm / qk-norm entry that no tuned kernel covers.
+ */
+enum {
+  DMF_ATTN_PLAN_FWD = 0,            /* dmf_attn_fwd                                  */
+  DMF_ATTN_PLAN_FWD_JVP = 1,        /* dmf_attn_fwd_jvp                              */
+  DMF_ATTN_PLAN_BWD = 2,            /* dmf_attn_bwd                                  */
+  DMF_ATTN_PLAN_FWD_QNORM_JVP = 3,  /* dmf_attn_fwd_qnorm / _qknorm without k_gain   */
+  DMF_ATTN_PLAN_FWD_QKNORM_JVP = 4  /* dmf_attn_fwd_qknorm with k_gain, with tangents */
+};
+DMF_ATTN_API int dmf_attn_plan(int entry, int B, int H, int Lq, int Lkv, int D, int dtype,
+                  char* buf, int buflen);
+
 #ifdef __cplusplus
 }
 #endif

@@ -89,6 +89,11 @@ def test_model_call_shapes_take_the_narrow_work_groups(B, H, D):
     head dim 64, the backward launcher the kernel pair.  Sampled (batch, head) units against the oracle, and the
     fused forward against the primal-only one, which keeps 256-row work-groups."""
     L, dtype, scale = 256, torch.bfloat16, D ** -0.5
+    # the launch policies depend on the device's compute-unit count: make sure this device takes the paths named above
+    assert _lib.plan("fwd_jvp", B, H, L, L, D) == f"dmf::attn_fwd_bf16_kernel<{D}, true, 4, false, false>"
+    assert _lib.plan("fwd", B, H, L, L, D) == f"dmf::attn_fwd_bf16_kernel<{D}, false, 8, false, false>"
+    assert _lib.plan("bwd", B, H, L, L, D) == (f"dmf::attn_bwd_dq_bf16_kernel<64, 2> + dmf::attn_bwd_dkv_bf16_kernel<64, 4>" if D == 64
+                                                else f"dmf::attn_bwd_fused_bf16_kernel<{D}>")
     g = torch.Generator(device=DEV).manual_seed(B + D)
     q, k, v, tq, tk, tv, do = (torch.randn(B, L, H, D, generator=g, device=DEV).to(dtype) for _ in range(7))
     o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)[:3]

@@ -21,6 +21,21 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout) and not r.stdout.strip().startswith("{")
 
 
+def test_offline_counter_rows_belong_to_the_kernels_in_this_tree():
+    """The traffic / MFMA-busy figures bench.py quotes were measured offline; each row carries the kernel name and the
+    hash of the kernel source it was taken on, and bench.py withholds a row that no longer matches.  The committed
+    tree must not be in that state (on a 256-CU device, which is also what the host-only plan query assumes here)."""
+    sys.path.insert(0, ROOT)
+    import bench
+    from dmf_amd import _lib
+    for (kind, wname), row in bench.OFFLINE_COUNTERS.items():
+        B, H, N, D, _ = bench.WORKLOADS[wname]
+        assert row["kernel"] == _lib.plan(kind, B, H, N, N, D), (kind, wname)
+        assert row["src"][1] == bench.source_hash(row["src"][0]), f"{kind} {wname}: counters were measured on an older {row['src'][0]}"
+        text = open(os.path.join(ROOT, bench.PROFILE_FILES[(kind, wname)])).read()
+        assert all(k in text for k in row["kernel"].split(" + ")), bench.PROFILE_FILES[(kind, wname)]
+
+
 @pytest.mark.gpu
 def test_json_line_contract():
     r = _run("--steps", "6", "--warmup", "2", "--no-extra")

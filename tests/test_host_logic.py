@@ -29,7 +29,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = _declared_symbols()
-    assert len(names) == 21 and set(names) == set(_lib.SIGNATURES), names
+    assert len(names) == 22 and set(names) == set(_lib.SIGNATURES), names
     for n in names:
         assert getattr(lib, n) is not None
     assert lib.dmf_attn_version() >= 1
@@ -37,6 +37,28 @@ def test_library_exports_every_declared_symbol():
     for code in range(-9, 0):
         assert b"unknown" not in lib.dmf_attn_strerror(code)
     assert b"unknown" in lib.dmf_attn_strerror(-99)
+
+
+def test_plan_names_the_kernels_without_launching():
+    """dmf_attn_plan is host-only: it answers on a machine without a GPU too (a device whose compute-unit count cannot
+    be asked counts as 256 units, the MI355X's)."""
+    bf, f32 = torch.bfloat16, torch.float32
+    assert _lib.plan("fwd_jvp", 64, 16, 1024, 1024, 72, bf) == "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>"
+    assert _lib.plan("fwd", 256, 16, 256, 256, 72, bf) == "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>"
+    assert _lib.plan("bwd", 256, 16, 256, 256, 72, bf) == "dmf::attn_bwd_fused_bf16_kernel<72>"
+    assert _lib.plan("bwd", 64, 16, 1024, 1024, 72, bf) == "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72, 4>"
+    assert _lib.plan("bwd", 2, 2, 128, 128, 72, bf).startswith("dmf::attn_bwd_dq_bf16_kernel")     # too short for the single pass
+    assert _lib.plan("fwd_jvp", 2, 12, 256, 256, 64, f32) == "dmf::attn_fwd_kernel<float, 64, true>"
+    assert _lib.plan("fwd", 1, 1, 7, 9, 32, bf) == "dmf::attn_fwd_kernel<__bf16, 32, false>"            # no tuned kernel at head dim 32
+    assert _lib.plan("fwd_qknorm_jvp", 16, 16, 1024, 1024, 72, bf) == "dmf::attn_fwd_bf16_kernel<72, true, 8, true, true>"
+    with pytest.raises(RuntimeError, match="no kernel"):
+        _lib.plan("fwd_qnorm_jvp", 1, 1, 64, 64, 72, f32)
+    lib = _lib.load()
+    small = ctypes.create_string_buffer(8)
+    assert lib.dmf_attn_plan(1, 1, 1, 64, 64, 72, 1, small, 8) == 0 and small.value == b"dmf::at"   # truncated, NUL-terminated
+    assert lib.dmf_attn_plan(1, 1, 1, 64, 64, 40, 1, small, 8) == -2
+    assert lib.dmf_attn_plan(9, 1, 1, 64, 64, 72, 1, small, 8) == -3
+    assert lib.dmf_attn_plan(1, 1, 1, 64, 64, 72, 1, None, 8) == -5
 
 
 def test_validation_codes_without_launch():
@@ -317,6 +339,9 @@ def test_stale_gradient_accumulator_probe():
     from dmf_amd.harness import stale_grad_accumulator
     p = torch.nn.Parameter(torch.randn(3))
     assert not stale_grad_accumulator(p) and not stale_grad_accumulator(p)
+    with torch.no_grad():                      # the probe must not depend on the caller's gradient mode
+        assert not stale_grad_accumulator(p)
+    assert not stale_grad_accumulator(torch.zeros(3))   # no gradient, no accumulator
     loss = (p * 2).sum()
     assert stale_grad_accumulator(p)
     loss.backward()
