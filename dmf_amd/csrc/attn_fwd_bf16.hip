@@ -49,6 +49,11 @@ struct FastCfg {
   static constexpr int PAD_IDX = 4 * ((D % 32) / 8) + (D % 4);             // 32-wide last tile: accumulator element holding row D%32 ...
   static constexpr int PAD_G = ((D % 32) % 8) / 4;                         // ... in the lanes of this half
   static constexpr int PAD16_ROW = (D % 32) / 4, PAD16_E = D % 4;          // 16-wide tail: lanes of 16-lane row PAD16_ROW, element PAD16_E
+  // Spare contraction slots in the last score chunk (head dim 72: slots 72..79 of 5 x 16): slots D..D+2 carry the running
+  // maximum -- Q's pad elements hold -m as a bf16 triple (hi + mid + lo, 2^-24 relative) against ones in the K rows, and Q
+  // is pre-multiplied by scale*log2(e) -- so that the MFMAs deliver S*log2(e) - m and the exponentials take their argument
+  // as it is (no multiply-add per score).
+  static constexpr bool MFOLD = 2 * NCHUNK > VPR;
 };
 
 // NW = waves per work-group: 4 (128 query rows, two work-groups per CU) or
@@ -116,7 +121,8 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   for (int s = 0; s < 2; ++s) {
     for (int i = tid; i < BKV * (KP - VPR); i += NTHR) {
       const int off = ((i / (KP - VPR)) * KP + VPR + i % (KP - VPR)) * 16;
-      *reinterpret_cast<u32x4*>(Kt(s) + off) = u32x4{0, 0, 0, 0};
+      const bool one = F::MFOLD && i % (KP - VPR) == 0;   // elements D..D+2 of a K row = 1.0 (bf16 0x3f80): they multiply the -m triple in Q's pad slots
+      *reinterpret_cast<u32x4*>(Kt(s) + off) = u32x4{one ? 0x3f803f80u : 0u, one ? 0x3f80u : 0u, 0, 0};
       if constexpr (JVP) *reinterpret_cast<u32x4*>(dKt(s) + off) = u32x4{0, 0, 0, 0};
     }
     if constexpr (VP > VPR) {
@@ -130,8 +136,10 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
     }
   }
 
-  // ---- Q, dQ operand chunks, pre-multiplied by the softmax scale
-  u32x4 Qr[NCHUNK], dQr[JVP ? NCHUNK : 1];
+  // ---- Q, dQ operand chunks, pre-multiplied by the softmax scale.  MFOLD: the score product takes QrS = q*scale*log2(e)
+  //      (+ the pad slot), the dK product of the tangent scores still Qr = q*scale (kept only with tangents).
+  constexpr bool MFOLD = F::MFOLD;
+  u32x4 Qr[NCHUNK], dQr[JVP ? NCHUNK : 1], QrS[MFOLD ? NCHUNK : 1], mB = {0, 0, 0, 0};
   {
     const int qrow = q0 + wave * 32 + c32;
     const uint32_t rb_q = (uint32_t)p.st[0][1] * 2;
@@ -230,8 +238,26 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
       for (int e = 0; e < 4; ++e) y[e] = pack_bf16x2(lo(x[e]) * p.scale, hi(x[e]) * p.scale);
       return y;
     };
+    // MERGE (tangents, half-empty last chunk): the two last-chunk products of the tangent scores, K dQ^T and dK Q^T over
+    // head-dim columns 16(NCHUNK-1) .., fill half of the contraction slots each; they are issued as ONE MFMA whose A
+    // operand takes K in the lower half of the slots and dK in the upper half (a per-lane LDS address) against
+    // mB = [dQ | Q] -- one MFMA and one LDS read fewer per tile.
+    constexpr bool MERGE = JVP && 2 * NCHUNK > VPR;
+    if constexpr (MERGE) {
+      auto sc = [&](uint32_t w) { return pack_bf16x2(lo(w) * p.scale, hi(w) * p.scale); };
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t qs = sc(Qr[NCHUNK - 1][e]);
+        auto r = __builtin_amdgcn_permlane32_swap(qs, qs, false, false);   // r[0] of a lane above 31 = the value of lane - 32
+        mB[e] = g ? r[0] : sc(dQr[NCHUNK - 1][e]);
+      }
+    }
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
+      if constexpr (MFOLD) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) QrS[c][e] = pack_bf16x2(lo(Qr[c][e]) * p.scale_log2, hi(Qr[c][e]) * p.scale_log2);
+      }
       Qr[c] = scaled(Qr[c]);
       if constexpr (JVP) dQr[c] = scaled(dQr[c]);
     }
@@ -254,12 +280,15 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
     O16[hq] = f32x4{0, 0, 0, 0};
     dO16[hq] = f32x4{0, 0, 0, 0};
   }
-  float m_run = -INFINITY, l_run = 0.f, mu_run = 0.f;   // log2-domain running max; VALU row sums only when !PADROW
+  float m_run = F::MFOLD ? 0.f : -INFINITY, l_run = 0.f, mu_run = 0.f;   // log2-domain running max; VALU row sums only when !PADROW
 
   // Lane address for the transposed V / dV operand reads (see lds_col_operand):
   // 16 lanes fetch a 4-row x 16-column block, lane i supplying row i/4, columns 4*(i%4)..+3.
   constexpr int DV_OFF = F::KBYTES + F::VBYTES;   // dV tile sits this many bytes after the V tile
   const uint32_t k_lane_addr = lds_addr(smem) + c32 * KSTR * 2 + g * 16;   // row-operand reads of K / dK
+  // merged last tangent-score chunk: K's last valid vector for the lower half of the wave, dK's for the upper half
+  constexpr bool MERGE = JVP && 2 * NCHUNK > VPR;
+  const uint32_t m_lane_addr = lds_addr(smem) + c32 * KSTR * 2 + (VPR - 1) * 16 + g * (F::KBYTES + F::VBYTES);
   const uint32_t v_lane_addr =
       lds_addr(smem) + F::KBYTES + ((4 * g + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
   // Remainder (16x16x32) operand: 16-lane row w covers keys 16*(w%2) + 4*(w/2) + {0..3, 8..11} -- the keys whose
@@ -276,12 +305,12 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   const int ntiles = (p.Lkv + BKV - 1) / BKV;
   for (int it = 0; it < ntiles; ++it) {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's share of tile `it` has landed in LDS
-    lds_barrier();                         // ... and everyone else's; also: all waves are done with the other stage
-    const bool fetch = it + 1 < ntiles;    // tile it + 1 goes into the other stage, in parts between the score MFMAs
     const int s = it & 1;
     if constexpr (KN) {
       // k_hat = k r g, dk_hat = (dk r + k dr) g with r = (mean k^2 + eps)^-1/2, dr = -r^3 mean(k dk): models/layers.py:39-42 and
       // its tangent, element for element the arithmetic of the stand-alone norm kernel; rounded to bf16 in place.
+      // A wave normalises exactly the rows that it fetched itself (issue_tile_rows: rows RPW*wave .. +RPW-1 of K and dK), so
+      // its own vmcnt wait is all it needs and the barrier below publishes the normalised rows: no second barrier.
       constexpr int RPW = 32 / NW;
       auto lo = [](uint32_t w) { return __uint_as_float(w << 16); };
       auto hi = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
@@ -325,9 +354,10 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
             *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(p.k_hat) + (((int64_t)b * p.Lkv + key) * p.H + h) * D + 8 * cv) = kn;
         }
       }
-      lds_barrier();
     }
 
+    lds_barrier();                         // ... and everyone else's; also: all waves are done with the other stage
+    const bool fetch = it + 1 < ntiles;    // tile it + 1 goes into the other stage, in parts between the score MFMAs
     // ---- S^T (already scaled) and dS^T; the LDS reads of chunk c+1 are in
     //      flight while the MFMAs of chunk c run
     f32x16 S = {0}, dS = {0};
@@ -341,16 +371,21 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
         constexpr bool more = c + 1 < NCHUNK;
         if constexpr (more) {
           kc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ka);
-          if constexpr (JVP) dkc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DV_OFF>(ka);
+          if constexpr (MERGE && c + 2 == NCHUNK) dkc[(c + 1) & 1] = lds_read128_issue<0>(m_lane_addr + s * STAGE);   // [K | dK], last vectors
+          else if constexpr (JVP) dkc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DV_OFF>(ka);
         }
         if constexpr (JVP) {
           lds_read128_wait<more ? 2 : 0>(kc[c & 1], dkc[c & 1]);
-          mma_chunk<T>(S, kc[c & 1], Qr[c]);
-          mma_chunk<T>(dS, kc[c & 1], dQr[c]);
-          mma_chunk<T>(dS, dkc[c & 1], Qr[c]);
+          mma_chunk<T>(S, kc[c & 1], MFOLD ? QrS[c] : Qr[c]);
+          if constexpr (MERGE && c + 1 == NCHUNK) {
+            mma_chunk<T>(dS, dkc[c & 1], mB);
+          } else {
+            mma_chunk<T>(dS, kc[c & 1], dQr[c]);
+            mma_chunk<T>(dS, dkc[c & 1], Qr[c]);
+          }
         } else {
           lds_read128_wait<more ? 1 : 0>(kc[c & 1]);
-          mma_chunk<T>(S, kc[c & 1], Qr[c]);
+          mma_chunk<T>(S, kc[c & 1], MFOLD ? QrS[c] : Qr[c]);
         }
         if constexpr (c < NPART) {
           if (fetch) issue_part(it + 1, cc);
@@ -367,10 +402,22 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
     float mx = fmaxf(S[0], S[1]);
 #pragma unroll
     for (int i = 2; i < 16; ++i) mx = fmaxf(mx, S[i]);
-    mx = xhalf_max(mx) * kLog2e;
-    if (__builtin_amdgcn_ballot_w64(mx > m_run + kLazyLog2) != 0) {
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2(m_run - m_new);
+    mx = MFOLD ? xhalf_max(mx) : xhalf_max(mx) * kLog2e;   // MFOLD: the scores arrive as S*log2(e) - m_run
+    if (MFOLD ? (it == 0 || __builtin_amdgcn_ballot_w64(mx > kLazyLog2) != 0) : __builtin_amdgcn_ballot_w64(mx > m_run + kLazyLog2) != 0) {
+      float m_new, alpha;
+      if constexpr (MFOLD) {
+        // The first tile sets the maximum whatever its sign (m_run starts at 0, not -inf: it is a product term); later it is
+        // only raised.  This tile's scores, formed against the old maximum, are shifted by hand.
+        m_new = it == 0 ? m_run + mx : fmaxf(m_run, m_run + mx);
+        const float shift = m_new - m_run;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[i] -= shift;
+        alpha = it == 0 ? 0.f : fast_exp2(-shift);          // (nothing accumulated yet behind the first tile)
+        if (g == 1) QrS[NCHUNK - 1] = split3_bf16(-m_new);
+      } else {
+        m_new = fmaxf(m_run, mx);
+        alpha = fast_exp2(m_run - m_new);
+      }
       m_run = m_new;
       if constexpr (!F::PADROW) {
         l_run *= alpha;
@@ -396,7 +443,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
     f32x16 E, G;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      E[i] = fast_exp2(fmaf(S[i], kLog2e, -m_run));
+      E[i] = MFOLD ? fast_exp2(S[i]) : fast_exp2(fmaf(S[i], kLog2e, -m_run));
       if constexpr (JVP) G[i] = E[i] * dS[i];
       if constexpr (!F::PADROW) {
         l_run += E[i];
