@@ -194,6 +194,10 @@ template <int N>
 __device__ __forceinline__ void lds_read128_wait(u32x4& a, u32x4& b) {
   asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(a), "+v"(b) : [n] "n"(N));
 }
+template <int N>
+__device__ __forceinline__ void lds_read128_wait(u32x4& a, u32x4& b, u32x4& c, u32x4& d) {
+  asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : [n] "n"(N));
+}
 __device__ __forceinline__ ColOperand tr_operand(const TrPair& a) {
   ColOperand r;
   r.v = u32x4{a.lo[0], a.lo[1], a.hi[0], a.hi[1]};

@@ -54,6 +54,11 @@ struct FastCfg {
   // is pre-multiplied by scale*log2(e) -- so that the MFMAs deliver S*log2(e) - m and the exponentials take their argument
   // as it is (no multiply-add per score).
   static constexpr bool MFOLD = 2 * NCHUNK > VPR;
+  // Head dim 128 with tangents needs more than 256 registers (four accumulator tile pairs, eight Q and dQ operand chunks):
+  // the last QPARK chunks of Q and dQ are parked in LDS (each wave its own lanes, written once) and read back next to the
+  // K / dK chunks they multiply, instead of being spilled to scratch memory (256-row work-groups only: two 128-row
+  // work-groups per CU have no LDS to spare for it).
+  static constexpr int QPARK_JVP = D == 128 ? 4 : 0;
 };
 
 // NW = waves per work-group: 4 (128 query rows, two work-groups per CU) or
@@ -72,6 +77,9 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
   // Staging of this work-group's Q (and dQ) rows behind the two tile stages, when 160 KB of LDS have room for it.
   constexpr int QP = F::QP, QS_OFF = 2 * STAGE + 512, QS_BYTES = 32 * NW * QP * 16;
   constexpr bool QLDS = NW == 8 && QS_OFF + (JVP ? 2 : 1) * QS_BYTES <= 160 * 1024;
+  constexpr int QPARK = JVP && NW == 8 ? F::QPARK_JVP : 0;                 // parked operand k of wave w: QX_OFF + ((k * NW + w) * 64 + lane) * 16
+  constexpr int QX_OFF = 2 * STAGE + 512;
+  static_assert(QPARK == 0 || !QLDS, "the parked operands use the space behind the tile stages");
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   auto Kt = [&](int s) { return smem + s * STAGE; };
@@ -261,7 +269,16 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
       Qr[c] = scaled(Qr[c]);
       if constexpr (JVP) dQr[c] = scaled(dQr[c]);
     }
+    if constexpr (QPARK > 0) {
+#pragma unroll
+      for (int k = 0; k < QPARK; ++k) {
+        char* px = smem + QX_OFF + ((2 * k * NW + wave) * 64 + lane) * 16;
+        *reinterpret_cast<u32x4*>(px) = Qr[NCHUNK - QPARK + k];
+        *reinterpret_cast<u32x4*>(px + NW * 64 * 16) = dQr[NCHUNK - QPARK + k];
+      }
+    }
   }
+  const uint32_t qx_lane_addr = lds_addr(smem) + QX_OFF + (wave * 64 + lane) * 16;
 
   // first key tile on its way (issued after the Q loads: measured faster than issuing it first)
   if constexpr (!QLDS) issue(0);
@@ -363,25 +380,36 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
     f32x16 S = {0}, dS = {0};
     {
       const uint32_t ka = k_lane_addr + s * STAGE;
-      u32x4 kc[2], dkc[2];
+      u32x4 kc[2], dkc[2], qx[2], dqx[2];
+      static_assert(QPARK < NCHUNK, "the first chunk's operands stay in registers");
       kc[0] = lds_read128_issue<0>(ka);
       if constexpr (JVP) dkc[0] = lds_read128_issue<DV_OFF>(ka);
       static_for<NCHUNK>([&](auto cc) {
         constexpr int c = decltype(cc)::value;
         constexpr bool more = c + 1 < NCHUNK;
+        constexpr bool parked = c >= NCHUNK - QPARK, next_parked = more && c + 1 >= NCHUNK - QPARK;
         if constexpr (more) {
           kc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1)>(ka);
           if constexpr (MERGE && c + 2 == NCHUNK) dkc[(c + 1) & 1] = lds_read128_issue<0>(m_lane_addr + s * STAGE);   // [K | dK], last vectors
           else if constexpr (JVP) dkc[(c + 1) & 1] = lds_read128_issue<32 * (c + 1) + DV_OFF>(ka);
+          if constexpr (next_parked) {
+            constexpr int k = c + 1 - (NCHUNK - QPARK);
+            qx[(c + 1) & 1] = lds_read128_issue<2 * k * NW * 64 * 16>(qx_lane_addr);
+            dqx[(c + 1) & 1] = lds_read128_issue<(2 * k + 1) * NW * 64 * 16>(qx_lane_addr);
+          }
         }
         if constexpr (JVP) {
-          lds_read128_wait<more ? 2 : 0>(kc[c & 1], dkc[c & 1]);
-          mma_chunk<T>(S, kc[c & 1], MFOLD ? QrS[c] : Qr[c]);
+          constexpr int newer = more ? (next_parked ? 4 : 2) : 0;   // reads issued since this chunk's
+          if constexpr (parked) lds_read128_wait<newer>(kc[c & 1], dkc[c & 1], qx[c & 1], dqx[c & 1]);
+          else lds_read128_wait<newer>(kc[c & 1], dkc[c & 1]);
+          const u32x4& qc = parked ? qx[c & 1] : Qr[c];
+          const u32x4& dqc = parked ? dqx[c & 1] : dQr[c];
+          mma_chunk<T>(S, kc[c & 1], MFOLD ? QrS[c] : qc);
           if constexpr (MERGE && c + 1 == NCHUNK) {
             mma_chunk<T>(dS, dkc[c & 1], mB);
           } else {
-            mma_chunk<T>(dS, kc[c & 1], dQr[c]);
-            mma_chunk<T>(dS, dkc[c & 1], Qr[c]);
+            mma_chunk<T>(dS, kc[c & 1], dqc);
+            mma_chunk<T>(dS, dkc[c & 1], qc);
           }
         } else {
           lds_read128_wait<more ? 1 : 0>(kc[c & 1]);
@@ -564,7 +592,9 @@ static int launch_fast_q(const FwdParams& p, int BH, hipStream_t stream) {
   constexpr int tiles = 2 * (JVP ? 2 : 1) * (F::KBYTES + F::VBYTES) + 512;
   constexpr int stage = 32 * NW * Cfg<__bf16, D>::OROWV * 16;
   constexpr int qst = (JVP ? 2 : 1) * 32 * NW * F::QP * 16;                       // Q / dQ staging of the 8-wave kernel (see QLDS there)
-  constexpr int need = (NW == 8 && tiles + qst <= 160 * 1024) ? tiles + qst : tiles;
+  constexpr int park = (JVP && NW == 8 ? F::QPARK_JVP : 0) * 2 * NW * 64 * 16;                 // parked Q / dQ operand chunks
+  constexpr int need = (NW == 8 && tiles + qst <= 160 * 1024) ? tiles + qst : tiles + park;
+  static_assert(need <= 160 * 1024, "LDS budget");
   constexpr int smem = need > stage ? need : stage;
   auto kern = attn_fwd_bf16_kernel<D, JVP, NW, QN, KN>;
   static bool lds_ok[64] = {};
