@@ -96,6 +96,14 @@ __device__ __forceinline__ void lds_write128_untracked(uint32_t addr, u32x4 w) {
   asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(w), "n"(OFF) : "memory");
 }
 
+// One transposed 8-byte LDS read issued as a raw instruction (see lds_tr16_issue in attn_common.h for the pair form).
+template <int OFF>
+__device__ __forceinline__ u32x2 lds_tr16_issue1(uint32_t lane_addr) {
+  u32x2 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(r) : "v"(lane_addr), "n"(OFF));
+  return r;
+}
+
 // 4-byte LDS read issued as a raw instruction; lgkmcnt must be waited for before the result is used.
 __device__ __forceinline__ uint32_t lds_read32_issue(uint32_t addr) {
   uint32_t r;
@@ -547,11 +555,13 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_bwd_dkv_bf16_kernel(cons
 // LDS: K (8 tiles) | NST stages of Q, dout tiles | X (64 KB, reused as store staging) | lse, delta of all rows.
 template <int D>
 struct BwdFusedCfg {
-  using F = BwdFastCfg<D>;
+  using F = BwdFastCfg<D, true>;
   static constexpr int TB = F::TBYTES;
   static constexpr int XBYTES = 65536, STATBYTES = 2 * 256 * 4;
-  // Q / dout stages: as many as the LDS has room for (4: tiles are requested three iterations ahead, which covers the
-  // HBM latency of a work-group that has the CU to itself)
+  // Q / dout stages: as many as the LDS has room for next to tiles of the pitch that keeps the transposed reads free of
+  // bank conflicts (head dims 72 and 80: three stages of 13-vector rows rather than four of 11, 1 % faster).  A third or
+  // fourth stage only has to absorb jitter: the wait for a tile's delta rows at the end of every iteration already leaves
+  // nothing but the newest tile request in flight, so a tile has two iterations to arrive whatever the depth.
   static constexpr int NST = (8 + 2 * 4) * TB + XBYTES + STATBYTES <= 160 * 1024 ? 4 : ((8 + 2 * 3) * TB + XBYTES + STATBYTES <= 160 * 1024 ? 3 : 2);
   static constexpr int K_OFF = 0, QS_OFF = 8 * TB, X_OFF = QS_OFF + 2 * NST * TB, STAT_OFF = X_OFF + XBYTES;
   static constexpr int LDS_BYTES = STAT_OFF + STATBYTES;
@@ -563,7 +573,7 @@ struct BwdFusedCfg {
 
 template <int D>
 __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdParams p) {
-  using F = BwdFastCfg<D>;
+  using F = BwdFastCfg<D, true>;
   using FC = BwdFusedCfg<D>;
   using T = __bf16;
   constexpr int VPR = F::VPR, NCHUNK = F::NCHUNK, NMT = F::NMT, P = F::P, STR = F::STR, TB = FC::TB;
@@ -610,38 +620,53 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
   //      lse and the first tile's dout / o rows (for delta), the first Q / dout tile, this wave's K and V rows, further
   //      tiles.
   // Every wave issues exactly two DMA instructions per Q / dout tile, and
-  // wait_tile(j) lets the ones issued after tile j stay in flight (vector memory operations complete in order, and
-  // anything not counted here can only make the wait stricter).
+  // wait_tile() -- called when tile j is needed -- lets the ones issued after tile j stay in flight (vector memory operations
+  // complete in order, and anything not counted here can only make the wait stricter).
   // Tiles 0 .. NST-2 are requested up front, then tile j+NST-1 at the top of iteration j: when tile j is waited for,
-  // the tiles j+1 .. j+NST-2 (as far as they exist) were requested after it.
+  // the tiles j+1 .. j+NST-2 were requested after it.
   auto issue_q = [&](int j) {   // tile j goes to stage j % NST
     char* st = smem + FC::QS_OFF + (j % NST) * STAGE;
     issue_tile_rows<P, VPR, 8>(rs_q, rb_q, (uint32_t)j * 32 * rb_q, st, wave, lane);
     issue_tile_rows<P, VPR, 8>(rs_do, rb_do, (uint32_t)j * 32 * rb_do, st + DO_OFF, wave, lane);
   };
-  auto wait_tile = [&](int j) {
-    const int newer = 2 * min(NST - 2, nqt - 1 - j);
-    if (newer >= 12) __builtin_amdgcn_s_waitcnt(0x0F7C);
-    else if (newer >= 8) __builtin_amdgcn_s_waitcnt(0x0F78);
-    else if (newer >= 4) __builtin_amdgcn_s_waitcnt(0x0F74);
-    else if (newer >= 2) __builtin_amdgcn_s_waitcnt(0x0F72);
-    else __builtin_amdgcn_s_waitcnt(0x0F70);
+  // Tiles past the end are requested like the others (every row is out of range: the bounds check zero-fills the stage
+  // and nothing reads it), so that the number of DMA instructions in flight behind any tile is a constant, 2 (NST - 2),
+  // and no wait depends on how many tiles are left.
+  auto wait_tile = [&]() {
+    static_assert(NST >= 2 && 2 * (NST - 2) <= 15, "vmcnt immediate");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (NST - 2)));
   };
+  // Work-group barrier with no fence attached: a release fence would make the compiler wait for every outstanding
+  // buffer_load ... lds (vmcnt(0)), i.e. for the tiles requested ahead.  This wave's own LDS traffic is waited for here;
+  // what a barrier publishes of the DMA data is decided by the explicit wait_tile() in front of it.
+  auto bare_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
   // delta = rowsum(dout * o) of the 32 query rows of a tile, by the whole work-group: 16 lanes per row, one 16-byte
   // vector of dout and of o per lane (lanes past the head dim read zeros), summed across the 16 lanes.
   const uint32_t rb_o = (uint32_t)p.st[4][1] * 2;
   const __amdgpu_buffer_rsrc_t rs_o = make_rows_rsrc(reinterpret_cast<const T*>(p.o) + base(4), rb_o, p.Lq, D * 2);
+  // The three loads of a delta request are raw instructions with an explicit wait (delta_wait): loads the compiler tracks
+  // would be waited for with vmcnt(0) / vmcnt(1) -- it does not count the tile DMA issued behind them -- i.e. together with
+  // the tile requested in the same iteration.  Every lane loads (no divergent branch around a raw load: the compiler could
+  // copy the destination register at the join before the data is there); lanes without a row read a clamped address.
   struct DeltaRows { u32x4 d, o; float lse; };
+  const u32x4 rsw_do = rows_rsrc_words(reinterpret_cast<const T*>(p.dout) + base(0), rb_do, p.Lq, D * 2);
+  const u32x4 rsw_o = rows_rsrc_words(reinterpret_cast<const T*>(p.o) + base(4), rb_o, p.Lq, D * 2);
   auto delta_request = [&](int j) {
     const int qrow = 32 * j + (tid >> 4), cv = tid & 15;
     DeltaRows r;
-    r.lse = 0.f;
-    if constexpr (SC) {
-      if (cv == 15 && qrow < p.Lq) r.lse = p.lse[(int64_t)bh * p.Lq + qrow];
-    }
-    r.d = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_do, cv < VPR ? (uint32_t)qrow * rb_do + cv * 16 : 0x7ffffff0u, 0, 0));
-    r.o = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_o, cv < VPR ? (uint32_t)qrow * rb_o + cv * 16 : 0x7ffffff0u, 0, 0));
+    const float* lp = p.lse + (int64_t)bh * p.Lq + min(qrow, p.Lq - 1);
+    asm volatile("global_load_dword %0, %1, off" : "=v"(r.lse) : "v"(lp));
+    const uint32_t vd = cv < VPR ? (uint32_t)qrow * rb_do + cv * 16 : 0x7ffffff0u, vo = cv < VPR ? (uint32_t)qrow * rb_o + cv * 16 : 0x7ffffff0u;
+    // (s_nop: a descriptor the compiler has just restored with v_readlane needs five wait states before a vector memory
+    //  instruction may read it, and the compiler does not look into the block for that)
+    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %2, %4, 0 offen\n\tbuffer_load_dwordx4 %1, %3, %5, 0 offen"
+                 : "=&v"(r.d), "=&v"(r.o)
+                 : "v"(vd), "v"(vo), "s"(rsw_do), "s"(rsw_o));
     return r;
+  };
+  // N = vector-memory instructions issued since the request that may stay in flight
+  auto delta_wait = [&](DeltaRows& r, auto nc) {
+    asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(r.d), "+v"(r.o), "+v"(r.lse) : [n] "n"(decltype(nc)::value));
   };
   auto delta_finish = [&](int j, const DeltaRows& r) {
     float s = 0.f;
@@ -662,9 +687,10 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
     if ((tid & 15) == 15) {
       const bool qok = qrow < p.Lq;
       if constexpr (SC) {   // rows past the end: P = 0 through a huge "lse"
-        char* row = smem + FC::QS_OFF + (j % NST) * STAGE + ((tid >> 4) * P + VPR) * 16;
-        *reinterpret_cast<u32x4*>(row) = split3_bf16(qok ? -r.lse * kLog2e : -1e30f);
-        *reinterpret_cast<u32x4*>(row + DO_OFF) = split3_bf16(qok ? -s : 0.f);
+        // (raw stores: in front of a store it tracks the compiler would wait for the tile DMA in flight)
+        const uint32_t row = lds_addr(smem) + FC::QS_OFF + (j % NST) * STAGE + ((tid >> 4) * P + VPR) * 16;
+        lds_write128_untracked<0>(row, split3_bf16(qok ? -r.lse * kLog2e : -1e30f));
+        lds_write128_untracked<DO_OFF>(row, split3_bf16(qok ? -s : 0.f));
       } else {
         stat_delta[qrow] = qok ? s : 0.f;
       }
@@ -682,8 +708,9 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
   //      before the first barrier (rows past Lkv read as zeros)
   issue_rows<P, VPR, 32>(rs_k, rb_k, (uint32_t)(wave * 32) * rb_k, smem + FC::K_OFF + wave * TB, lane);
   issue_rows<P, VPR, 32>(rs_v, rb_v, (uint32_t)(wave * 32) * rb_v, smem + FC::X_OFF + wave * TB, lane);
-  for (int j = 1; j < NST - 1 && j < nqt; ++j) issue_q(j);
-  wait_tile(0);   // loads complete in order: the key rows (and tile 0) have landed, the later tiles may still be in flight
+  for (int j = 1; j < NST - 1; ++j) issue_q(j);
+  wait_tile();    // loads complete in order: the key rows, tile 0 and the delta request have landed, the later tiles may still be in flight
+  delta_wait(dr, std::integral_constant<int, 2 * (NST - 2)>{});
   // ---- this lane's key row: V stays in registers for the whole kernel, K (times scale*log2e) is re-read from the LDS
   //      copy at the top of every half (so that its registers are free while dQ is formed)
   const int krow = wave * 32 + c32;
@@ -738,11 +765,11 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
     }
     for (int j = 4 * half; j < j_end; ++j) {
       if (j == 0 || j != 4 * half) {   // (the first tile of a later half was waited for before the dQ rows were stored)
-        wait_tile(j);     // this wave's share of tile j has landed
-        lds_barrier();    // ... and everyone else's; all waves are done with the stage of tile j-1
+        wait_tile();      // this wave's share of tile j has landed
+        bare_barrier();   // ... and everyone else's; all waves are done with the stage of tile j-1
       }
-      if (j + 1 < nqt) dr = delta_request(j + 1);   // (before the tile request: its data is wanted first)
-      if (j + NST - 1 < nqt) issue_q(j + NST - 1);
+      dr = delta_request(min(j + 1, nqt - 1));   // (before the tile request: its data is wanted first; behind the last tile: dropped)
+      issue_q(j + NST - 1);
       const uint32_t stage_off = FC::QS_OFF + (j % NST) * STAGE;
       const uint32_t ra = row_addr + stage_off, ca = lds_addr(smem) + col_off + stage_off;
 
@@ -870,10 +897,14 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
         });
       }
 #undef DMF_PIN
+      delta_wait(dr, std::integral_constant<int, 2>{});   // (this iteration's tile request may stay in flight)
       if (j + 1 < nqt) delta_finish(j + 1, dr);   // visible to the other waves after the next barrier
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's dS tiles are in LDS
-    lds_barrier();                                        // X holds every dS tile of this half
+    // This wave's dS tiles are in LDS, then everyone's: X holds every dS tile of this half.  A bare barrier: the fenced
+    // lds_barrier() would also wait for the Q / dout tile DMA in flight (vmcnt(0): a release fence covers the LDS writes of
+    // outstanding buffer_load ... lds instructions), about 2000 cycles per half, and nothing read below comes from a DMA
+    // that is still in flight (the K tiles landed before the first tile).
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
     // ================= phase 2: dQ^T = K^T dS^T for query tile jq, output tiles of this wave's part
     const int jq = 4 * half + (wave & 3);
@@ -882,7 +913,59 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
     f32x4 dQ16[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
 #pragma unroll
     for (int t = 0; t < NT0; ++t) dQ[t] = f32x16{0};
-    if (jq < nqt) {
+    if constexpr (NMT == 2) {
+      // Straight-line form (two output tiles, one per part): always all eight key blocks -- the K rows and the dS tiles of
+      // keys past the end are zeros -- fully unrolled, every operand read issued as a raw instruction one key block ahead
+      // with an explicit lgkmcnt wait, no branch between an issue and its wait.  (Read through the tracked intrinsics the
+      // first operand would make the compiler wait for the Q / dout tile DMA in flight, about 2000 cycles per half.)  Both
+      // parts run the remainder products; part 1 drops its copy (two 16x16x32 MFMAs per key block) rather than branch.
+      if (jq < nqt) {
+        const int i16 = lane & 15, piece = 4 * ((lane >> 4) & 1) + (i16 & 3), r0 = 4 * g + (i16 >> 2);
+        // lane address inside a swizzled exchange tile: key row r, query piece `piece` (cf. the writer's x_swz)
+        auto xoff = [&](int r) { return (uint32_t)(r * 32 + ((piece ^ ((r >> 2) & 7)) << 2)) * 2; };
+        const uint32_t xb = x_base + (wave & 3) * 8 * FC::XTILE;
+        const uint32_t x00 = xb + xoff(r0), x01 = xb + xoff(r0 + 8), x10 = xb + xoff(r0 + 16), x11 = xb + xoff(r0 + 24);
+        const uint32_t ka = lds_addr(smem) + FC::K_OFF + col_off + (part1 ? 64u : 0u);   // part 1: head-dim columns 32 .. 63
+        const uint32_t kta = lds_addr(smem) + FC::K_OFF + tail_off;
+        struct RawOps { u32x2 b0l, b0h, b1l, b1h; TrPair a0, a1, tl; };
+        constexpr int NRD = 8 + (TAIL ? 2 : 0);   // LDS instructions per key block
+        RawOps ro[2];
+        auto issue_kb = [&](auto kc_) {
+          constexpr int kb = decltype(kc_)::value;
+          RawOps& o = ro[kb & 1];
+          o.b0l = lds_tr16_issue1<kb * FC::XTILE>(x00);
+          o.b0h = lds_tr16_issue1<kb * FC::XTILE>(x01);
+          o.b1l = lds_tr16_issue1<kb * FC::XTILE>(x10);
+          o.b1h = lds_tr16_issue1<kb * FC::XTILE>(x11);
+          o.a0 = lds_tr16_issue<kb * TB, kb * TB + 8 * STR * 2>(ka);
+          o.a1 = lds_tr16_issue<kb * TB + 16 * STR * 2, kb * TB + 24 * STR * 2>(ka);
+          if constexpr (TAIL) o.tl = lds_tr16_issue<kb * TB, kb * TB + 8 * STR * 2>(kta);
+        };
+        issue_kb(std::integral_constant<int, 0>{});
+        static_for<8>([&](auto kc_) {
+          constexpr int kb = decltype(kc_)::value;
+          if constexpr (kb + 1 < 8) issue_kb(std::integral_constant<int, kb + 1>{});
+          RawOps& o = ro[kb & 1];
+          if constexpr (TAIL)
+            asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(o.b0l), "+v"(o.b0h), "+v"(o.b1l), "+v"(o.b1h), "+v"(o.a0.lo), "+v"(o.a0.hi),
+                         "+v"(o.a1.lo), "+v"(o.a1.hi), "+v"(o.tl.lo), "+v"(o.tl.hi) : [n] "n"(kb + 1 < 8 ? NRD : 0));
+          else
+            asm volatile("s_waitcnt lgkmcnt(%[n])" : "+v"(o.b0l), "+v"(o.b0h), "+v"(o.b1l), "+v"(o.b1h), "+v"(o.a0.lo), "+v"(o.a0.hi),
+                         "+v"(o.a1.lo), "+v"(o.a1.hi) : [n] "n"(kb + 1 < 8 ? NRD : 0));
+          ColOperand b0, b1;
+          b0.v = u32x4{o.b0l[0], o.b0l[1], o.b0h[0], o.b0h[1]};
+          b1.v = u32x4{o.b1l[0], o.b1l[1], o.b1h[0], o.b1h[1]};
+          mma_col<T>(dQ[0], tr_operand(o.a0), b0);
+          mma_col<T>(dQ[0], tr_operand(o.a1), b1);
+          if constexpr (TAIL) {
+            ColOperand d0, d1;
+            tail_operands(b0, b1, d0, d1);
+            mma16(dQ16[0], tr_operand(o.tl), d0);
+            mma16(dQ16[1], tr_operand(o.tl), d1);
+          }
+        });
+      }
+    } else if (jq < nqt) {
       // Operands through the tracked LDS-read intrinsics here, not the raw-instruction helpers of phase 1: those are
       // only safe in straight-line code (between the issue and the wait the compiler may copy the destination
       // registers, e.g. at a branch, and would copy stale data), and this loop branches on the wave's part.  The
@@ -975,8 +1058,8 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
     }
     // The next half's first Q / dout tile was requested a whole tile ago: wait for it here, before the dQ rows are
     // stored, so that the barrier below also publishes it and the next wait for memory comes a tile after the stores.
-    if (j_end < nqt) wait_tile(j_end);
-    lds_barrier();   // every wave has read its dS tiles: X becomes the staging area of this half's dQ rows
+    wait_tile();
+    bare_barrier();  // every wave has read its dS tiles: X becomes the staging area of this half's dQ rows
     {
       using C = Cfg<T, D>;
       T* stage = reinterpret_cast<T*>(smem + FC::X_OFF);
@@ -999,7 +1082,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
             store4<T>(srow + (NT0 + t) * 32 + jj * 8 + 4 * g, dQ[t][4 * jj] * p.scale, dQ[t][4 * jj + 1] * p.scale, dQ[t][4 * jj + 2] * p.scale,
                       dQ[t][4 * jj + 3] * p.scale);
       }
-      lds_barrier();
+      bare_barrier();   // (no fence: tiles of the next half are in flight)
       T* gdq = reinterpret_cast<T*>(p.dq) + base(5);
       for (int v = tid; v < 128 * VPR; v += 512) {
         const int row = v / VPR, cv = v % VPR, qrow = half * 128 + row;

@@ -422,6 +422,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* bas
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (nrows - 1) * row_bytes + row_payload_bytes, 0x00020000);
 }
 
+// The same descriptor as four plain words, for raw buffer instructions in inline assembly ("s" operand).
+__device__ __forceinline__ u32x4 rows_rsrc_words(const void* base, uint32_t row_bytes, int nrows, int row_payload_bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  return u32x4{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)((nrows - 1) * row_bytes + row_payload_bytes), 0x00020000u};
+}
+
 // Epilogue of the 16-wide remainder tiles (head dims 72, 80): lane (i = lane % 16,
 // w = lane / 16) holds head-dim columns 32*NMT + 4w .. +3 of row i (tile 0) and of
 // row 16 + i (tile 1) of this wave's 32 rows; value(hq, e) supplies the numbers.

@@ -621,11 +621,13 @@ static int launch_fast_t(const FwdParams& p, int BH, hipStream_t stream) {
 //     (B64 N1024 0.779 -> 0.749 ms, B256 N256 0.293 -> 0.269, B64 H12 N256 0.056 -> 0.048; smaller grids lose);
 //   * other head dims, N <= 256: 4 waves win only where 8-wave work-groups would run in two or three rounds
 //     (B32 H16: 0.0438 -> 0.0413 ms, B48: 0.070 -> 0.062) and lose 2-3 % from four rounds on;
-//   * without tangents the 8-wave kernel already fits twice per CU and is never slower.
+//   * without tangents the 8-wave kernel fits twice per CU and is slower only at head dim 64 on large grids.
 static bool fwd_wide_workgroups(int Lq, int D, bool jvp, int BH) {
   if (Lq <= 128) return false;
-  if (!jvp) return true;
   const int cus = compute_units();
+  // (without tangents only head dim 64 on a grid of at least eight narrow work-groups per CU prefers them:
+  //  B256 H16 N256 0.129 -> 0.123 ms, B64 N1024 0.331 -> 0.326; the DMFT-B/2 call B64 H12 N256 is equal either way)
+  if (!jvp) return !(D == 64 && (int64_t)BH * ((Lq + 127) / 128) >= 8 * (int64_t)cus);
   if (D == 64) return (int64_t)BH * ((Lq + 127) / 128) < 3 * (int64_t)cus;
   if (Lq <= 256) {
     const int64_t rounds = ((int64_t)BH * ((Lq + 255) / 256) + cus - 1) / cus;

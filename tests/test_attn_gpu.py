@@ -562,6 +562,25 @@ def test_fwd_qknorm_matches_separate_norms_and_oracle(shape, jvp):
     assert ao.rel_l2(o.float().cpu(), o_ref) <= TOL[torch.bfloat16]
 
 
+def test_fwd_qknorm_eps_zero_with_ragged_key_length():
+    """eps = 0 and a key length that is not a multiple of the 32-row tile: the zero-filled rows past the end of the last
+    tile have no norm (1 / sqrt(0)); the in-kernel k norm must leave them at zero instead of turning them into NaNs that
+    would reach the tangent through P * dS = 0 * NaN.  Against the stand-alone norm kernel followed by the plain kernel."""
+    B, Lq, Lkv, H, D = 2, 40, 77, 2, 72
+    g = torch.Generator().manual_seed(977)
+    mk = lambda L: torch.randn(B, L, H, D, generator=g).to(torch.bfloat16).to(DEV)
+    q, tq, k, tk, v, tv = mk(Lq), mk(Lq), mk(Lkv), mk(Lkv), mk(Lkv), mk(Lkv)
+    gq, gk = (1 + 0.3 * torch.randn(D, generator=g)).to(DEV), (1 + 0.3 * torch.randn(D, generator=g)).to(DEV)
+    scale = D ** -0.5
+    o, to, lse, _, kh = _lib.fwd_qknorm(q, k, v, tq, tk, tv, gq, gk, 0.0, scale, save_normed=True)
+    assert all(bool(torch.isfinite(t.float()).all()) for t in (o, to, lse, kh))
+    qn, tqn = _lib.rmsnorm_fwd(q, gq, tq, 0.0, True)
+    kn, tkn = _lib.rmsnorm_fwd(k, gk, tk, 0.0, True)
+    o2, to2, lse2 = _lib.fwd_jvp(qn, kn, v, tqn, tkn, tv, scale)
+    assert torch.equal(kh, kn)
+    assert ao.rel_l2(o.float(), o2.float()) <= 3e-3 and ao.rel_l2(to.float(), to2.float()) <= 3e-3 and ao.rel_l2(lse, lse2) <= 1e-3
+
+
 @pytest.mark.parametrize("L", [264, 1024, 256, 77])
 def test_qknorm_qkvpacked_in_kernel_norms_forward_and_backward_vs_oracle(L, monkeypatch):
     """The packed q/k-norm + attention node on the tuned path.  Up to 256 rows the forward is ONE attention launch on
