@@ -163,6 +163,17 @@ def test_ragged_lengths(Lq, Lkv, dtype):
     _parity(2, Lq, 2, 72, dtype, seed=Lq * 7 + Lkv, Lkv=Lkv)
 
 
+@pytest.mark.parametrize("D", [64, 72, 80, 96])
+@pytest.mark.parametrize("Lq,Lkv", [(256, 256), (20, 256), (256, 20), (97, 250), (250, 97), (129, 129), (160, 33)])
+def test_single_pass_backward_every_head_dim_and_short_sides(Lq, Lkv, D):
+    """The one-work-group-per-head backward at every head dim it serves (each has its own tile pitch, stage count and dQ
+    phase), with one query tile, one key block, and lengths that leave the last tile, the last half and whole key
+    blocks partly or entirely empty (requests past the end are issued and zero-filled by design)."""
+    B, H = 2, 2
+    assert _lib.plan("bwd", B, H, Lq, Lkv, D, torch.bfloat16) == f"dmf::attn_bwd_fused_bf16_kernel<{D}>"
+    _parity(B, Lq, H, D, torch.bfloat16, seed=Lq + 3 * Lkv + D, Lkv=Lkv)
+
+
 @pytest.mark.parametrize("L", [200, 300, 1024])
 def test_peaked_softmax_inputs(L):
     """Inputs of twice the contract's scale: logits up to +-30, |lse| up to 25 -- the range in which the statistics folded
