@@ -643,7 +643,6 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
   // delta = rowsum(dout * o) of the 32 query rows of a tile, by the whole work-group: 16 lanes per row, one 16-byte
   // vector of dout and of o per lane (lanes past the head dim read zeros), summed across the 16 lanes.
   const uint32_t rb_o = (uint32_t)p.st[4][1] * 2;
-  const __amdgpu_buffer_rsrc_t rs_o = make_rows_rsrc(reinterpret_cast<const T*>(p.o) + base(4), rb_o, p.Lq, D * 2);
   // The three loads of a delta request are raw instructions with an explicit wait (delta_wait): loads the compiler tracks
   // would be waited for with vmcnt(0) / vmcnt(1) -- it does not count the tile DMA issued behind them -- i.e. together with
   // the tile requested in the same iteration.  Every lane loads (no divergent branch around a raw load: the compiler could
