@@ -41,13 +41,13 @@ HBM_PEAK_GBS = 8000.0
 # q, k, v, dout twice.
 OFFLINE_COUNTERS = {
     ("fwd_jvp", "xl2_512px"): {"traffic": 1.2124e+09, "mfma_busy": 0.596, "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>",
-                               "src": ("attn_fwd_bf16.hip", "497f13eebfbe383d")},
+                               "src": ("attn_fwd_bf16.hip", "8b80f746688ed301")},
     ("fwd_jvp", "xl2_256px"): {"traffic": 1.2124e+09, "mfma_busy": 0.351, "kernel": "dmf::attn_fwd_bf16_kernel<72, true, 8, false, false>",
-                               "src": ("attn_fwd_bf16.hip", "497f13eebfbe383d")},
+                               "src": ("attn_fwd_bf16.hip", "8b80f746688ed301")},
     ("fwd", "xl2_512px"): {"traffic": 6.0848e+08, "mfma_busy": 0.529, "kernel": "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>",
-                           "src": ("attn_fwd_bf16.hip", "497f13eebfbe383d")},
+                           "src": ("attn_fwd_bf16.hip", "8b80f746688ed301")},
     ("fwd", "xl2_256px"): {"traffic": 6.0900e+08, "mfma_busy": 0.299, "kernel": "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>",
-                           "src": ("attn_fwd_bf16.hip", "497f13eebfbe383d")},
+                           "src": ("attn_fwd_bf16.hip", "8b80f746688ed301")},
     ("bwd", "xl2_512px"): {"traffic": 1.8711e+09, "mfma_busy": 0.514,
                            "kernel": "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72, 4>", "src": ("attn_bwd_bf16.hip", "97b83c9d41ecdcb7")},
     ("bwd", "xl2_256px"): {"traffic": 1.2168e+09, "mfma_busy": 0.227, "kernel": "dmf::attn_bwd_fused_bf16_kernel<72>",

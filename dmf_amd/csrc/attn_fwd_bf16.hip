@@ -382,6 +382,11 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
       const uint32_t ka = k_lane_addr + s * STAGE;
       u32x4 kc[2], dkc[2], qx[2], dqx[2];
       static_assert(QPARK < NCHUNK, "the first chunk's operands stay in registers");
+      // Q operand of the score product: the copy pre-multiplied by scale * log2e where the maximum rides in the MFMA
+      auto score_q = [&](auto cc, const u32x4& plain) -> const u32x4& {
+        if constexpr (MFOLD) return QrS[decltype(cc)::value];
+        else return plain;
+      };
       kc[0] = lds_read128_issue<0>(ka);
       if constexpr (JVP) dkc[0] = lds_read128_issue<DV_OFF>(ka);
       static_for<NCHUNK>([&](auto cc) {
@@ -404,7 +409,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
           else lds_read128_wait<newer>(kc[c & 1], dkc[c & 1]);
           const u32x4& qc = parked ? qx[c & 1] : Qr[c];
           const u32x4& dqc = parked ? dqx[c & 1] : dQr[c];
-          mma_chunk<T>(S, kc[c & 1], MFOLD ? QrS[c] : qc);
+          mma_chunk<T>(S, kc[c & 1], score_q(cc, qc));
           if constexpr (MERGE && c + 1 == NCHUNK) {
             mma_chunk<T>(dS, dkc[c & 1], mB);
           } else {
@@ -413,7 +418,7 @@ __global__ __launch_bounds__(64 * NW, 8 / NW) void attn_fwd_bf16_kernel(const Fw
           }
         } else {
           lds_read128_wait<more ? 1 : 0>(kc[c & 1]);
-          mma_chunk<T>(S, kc[c & 1], MFOLD ? QrS[c] : Qr[c]);
+          mma_chunk<T>(S, kc[c & 1], score_q(cc, Qr[c]));
         }
         if constexpr (c < NPART) {
           if (fetch) issue_part(it + 1, cc);
