@@ -1134,14 +1134,14 @@ static int launch_bwd_fast_t(const BwdParams& p, int BH, hipStream_t stream) {
 }
 
 // Policy: does the single-pass kernel take this case?  Whole (batch, head) units per work-group, every score tile formed
-// once.  (Head dim 64: the two kernels need 124 / 166 registers and are resident four / three work-groups per CU; from one
-// (batch, head) unit per CU on they are as fast as the single pass or faster -- B32 H12 N256 0.048 -> 0.042 ms,
-// B128 0.161 -> 0.150, B256 H16 equal -- and only a grid smaller than the device loses, 0.025 -> 0.029 at B16 H12.
-// Head dim 128: K, the tile stages and the exchange area exceed the LDS.)
-bool bwd_single_pass(int Lq, int Lkv, int D, int BH) {
+// once: 5 GEMM units where the kernel pair executes 7.  That also decides head dim 64, where the pair (124 / 166 registers,
+// four / three work-groups per CU) is the faster schedule -- on all-zero operands B256 H16 N256 0.278 ms against 0.299 -- but
+// both run into the package-power limit on data and the one that executes less wins: 0.40 -> 0.35 ms there,
+// 0.085 -> 0.071 at B64 H12, 0.045 -> 0.043 at B32 H12, 0.0216 -> 0.0207 at B8 H16.
+// (Head dim 128: K, the tile stages and the exchange area exceed the LDS.)
+bool bwd_single_pass(int Lq, int Lkv, int D, int /*BH*/) {
   const int Lmax = std::max(Lq, Lkv);
   if (D != 64 && D != 72 && D != 80 && D != 96) return false;
-  if (D == 64 && BH >= compute_units()) return false;
   return Lmax >= kFusedMinRows && Lmax <= kFusedMaxRows;
 }
 

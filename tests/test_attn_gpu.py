@@ -90,15 +90,15 @@ def test_xl2_shape_reduced_batch(L, dtype):
 @pytest.mark.parametrize("B,H,D", [(32, 16, 72), (64, 12, 64)])
 def test_model_call_shapes_take_the_narrow_work_groups(B, H, D):
     """The attention calls of DMFT-XL/2 at batch 32 and DMFT-B/2 at batch 64 (N = 256): grids for which the forward
-    launcher picks 128-row work-groups with tangents (two or three rounds of 256-row ones, resp. head dim 64) and, at
-    head dim 64, the backward launcher the kernel pair.  Sampled (batch, head) units against the oracle, and the
+    launcher picks 128-row work-groups with tangents (two or three rounds of 256-row ones, resp. head dim 64) and the
+    backward launcher the single-pass kernel.  Sampled (batch, head) units against the oracle, and the
     fused forward against the primal-only one, which keeps 256-row work-groups."""
     L, dtype, scale = 256, torch.bfloat16, D ** -0.5
     # the launch policies depend on the device's compute-unit count: make sure this device takes the paths named above
     assert _lib.plan("fwd_jvp", B, H, L, L, D) == f"dmf::attn_fwd_bf16_kernel<{D}, true, 4, false, false>"
     assert _lib.plan("fwd", B, H, L, L, D) == f"dmf::attn_fwd_bf16_kernel<{D}, false, 8, false, false>"
-    assert _lib.plan("bwd", B, H, L, L, D) == (f"dmf::attn_bwd_dq_bf16_kernel<64, 2> + dmf::attn_bwd_dkv_bf16_kernel<64, 4>" if D == 64
-                                                else f"dmf::attn_bwd_fused_bf16_kernel<{D}>")
+    assert _lib.plan("bwd", B, H, L, L, D) == f"dmf::attn_bwd_fused_bf16_kernel<{D}>"
+    assert _lib.plan("bwd", B, H, 128, 128, D) == f"dmf::attn_bwd_dq_bf16_kernel<{D}, 2> + dmf::attn_bwd_dkv_bf16_kernel<{D}, 4>"
     g = torch.Generator(device=DEV).manual_seed(B + D)
     q, k, v, tq, tk, tv, do = (torch.randn(B, L, H, D, generator=g, device=DEV).to(dtype) for _ in range(7))
     o, to, lse = _lib.fwd_jvp(q, k, v, tq, tk, tv, scale)[:3]
