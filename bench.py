@@ -48,10 +48,10 @@ OFFLINE_COUNTERS = {
                            "src": ("attn_fwd_bf16.hip", "8b80f746688ed301")},
     ("fwd", "xl2_256px"): {"traffic": 6.0900e+08, "mfma_busy": 0.299, "kernel": "dmf::attn_fwd_bf16_kernel<72, false, 8, false, false>",
                            "src": ("attn_fwd_bf16.hip", "8b80f746688ed301")},
-    ("bwd", "xl2_512px"): {"traffic": 1.8711e+09, "mfma_busy": 0.514,
-                           "kernel": "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72, 4>", "src": ("attn_bwd_bf16.hip", "1b33c1f34142771b")},
-    ("bwd", "xl2_256px"): {"traffic": 1.2168e+09, "mfma_busy": 0.227, "kernel": "dmf::attn_bwd_fused_bf16_kernel<72>",
-                           "src": ("attn_bwd_bf16.hip", "1b33c1f34142771b")},
+    ("bwd", "xl2_512px"): {"traffic": 1.8709e+09, "mfma_busy": 0.515,
+                           "kernel": "dmf::attn_bwd_dq_bf16_kernel<72, 2> + dmf::attn_bwd_dkv_bf16_kernel<72, 4>", "src": ("attn_bwd_bf16.hip", "0baa6add1e385c9d")},
+    ("bwd", "xl2_256px"): {"traffic": 1.2167e+09, "mfma_busy": 0.231, "kernel": "dmf::attn_bwd_fused_bf16_kernel<72>",
+                           "src": ("attn_bwd_bf16.hip", "0baa6add1e385c9d")},
 }
 
 

@@ -668,12 +668,21 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
     asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(r.d), "+v"(r.o), "+v"(r.lse) : [n] "n"(decltype(nc)::value));
   };
   auto delta_finish = [&](int j, const DeltaRows& r) {
+    // Packed bf16 dot products with fp32 accumulation: four instructions for the eight products instead of sixteen
+    // unpacks and eight multiply-adds (the tile loop is bound by the instructions it issues).  The dot instructions have a
+    // longer pipeline than other VALU operations: chained through their accumulator they need no wait, but an ordinary
+    // VALU instruction that reads the result needs three wait states, which the compiler does not insert for a block it
+    // cannot look into -- hence the s_nop behind it (and one in front, for the accumulator's initial value).
     float s = 0.f;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      s += __uint_as_float(r.d[e] << 16) * __uint_as_float(r.o[e] << 16);
-      s += __uint_as_float(r.d[e] & 0xffff0000u) * __uint_as_float(r.o[e] & 0xffff0000u);
-    }
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_dot2c_f32_bf16 %0, %1, %5\n\t"
+        "v_dot2c_f32_bf16 %0, %2, %6\n\t"
+        "v_dot2c_f32_bf16 %0, %3, %7\n\t"
+        "v_dot2c_f32_bf16 %0, %4, %8\n\t"
+        "s_nop 3"
+        : "+v"(s)
+        : "v"(r.d[0]), "v"(r.d[1]), "v"(r.d[2]), "v"(r.d[3]), "v"(r.o[0]), "v"(r.o[1]), "v"(r.o[2]), "v"(r.o[3]));
     // inclusive sum over the row of 16 lanes (DPP row_shr 1, 2, 4, 8; lanes shifted in from outside read 0): lane 15 holds it
     auto shr = [](float x, auto n) {
       return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x110 + decltype(n)::value, 0xf, 0xf, true));
@@ -688,7 +697,9 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
       if constexpr (SC) {   // rows past the end: P = 0 through a huge "lse"
         // (raw stores: in front of a store it tracks the compiler would wait for the tile DMA in flight)
         const uint32_t row = lds_addr(smem) + FC::QS_OFF + (j % NST) * STAGE + ((tid >> 4) * P + VPR) * 16;
-        lds_write128_untracked<0>(row, split3_bf16(qok ? -r.lse * kLog2e : -1e30f));
+        u32x4 lv = split3_bf16(qok ? -r.lse * kLog2e : -1e30f);
+        lv[1] |= 0xF14A0000u;   // fourth pad element: -1e30 (bf16), met by a one only in the K rows of keys past the end
+        lds_write128_untracked<0>(row, lv);
         lds_write128_untracked<DO_OFF>(row, split3_bf16(qok ? -s : 0.f));
       } else {
         stat_delta[qrow] = qok ? s : 0.f;
@@ -760,7 +771,9 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) Kr[c] = scale_bf16x8(Kr[c], p.scale_log2);
     if constexpr (SC) {
-      if (g == 1) Kr[NCHUNK - 1] = ones3_bf16();
+      // (keys past the end: a fourth one against the -1e30 that every Q row carries in that slot, so that their P, and
+      //  with it their dS, is exactly zero without a select in the tile loop)
+      if (g == 1) Kr[NCHUNK - 1] = kvalid ? ones3_bf16() : u32x4{0x3f803f80u, 0x3f803f80u, 0u, 0u};
     }
     for (int j = 4 * half; j < j_end; ++j) {
       if (j == 0 || j != 4 * half) {   // (the first tile of a later half was waited for before the dQ rows were stored)
@@ -802,10 +815,11 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_fused_bf16_kernel(const BwdPa
         for (int e = 0; e < 4; ++e) dS[4 * jj + e] = Pm[4 * jj + e] * (SC ? dP[4 * jj + e] : dP[4 * jj + e] - __uint_as_float(d4[e]));
         if constexpr (jj & 1) {
           ds[jj >> 1] = acc_operand<T>(dS, jj >> 1);
-          // dS tile -> X (zeros for keys past the end: their K rows must not reach dQ)
+          // dS tile -> X (zeros for keys past the end: their K rows -- not zero-filled when the rows of a broadcast operand
+          // alias -- must not reach dQ; with SC their P is zero already, see the K operand above)
           static_for<2>([&](auto hc) {
             constexpr int q4 = jj - 1 + decltype(hc)::value;   // queries 8 q4 + 4g .. +3 of key row c32
-            const u32x2 w = kvalid ? u32x2{ds[q4 >> 1].v[2 * (q4 & 1)], ds[q4 >> 1].v[2 * (q4 & 1) + 1]} : u32x2{0, 0};
+            const u32x2 w = SC || kvalid ? u32x2{ds[q4 >> 1].v[2 * (q4 & 1)], ds[q4 >> 1].v[2 * (q4 & 1) + 1]} : u32x2{0, 0};
             lds_write64_untracked<0>(xa + (((2 * q4 + g) ^ x_swz) << 3), w);
           });
         }
