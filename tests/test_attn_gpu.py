@@ -293,6 +293,34 @@ def test_backward_with_broadcast_gradient(Lq, Lkv):
         _check(name + " (autograd)", got, exp.float().cpu(), 1e-6)
 
 
+@pytest.mark.parametrize("D", [64, 72, 128])
+@pytest.mark.parametrize("Lq,Lkv", [(256, 200), (150, 130), (300, 290)])
+def test_broadcast_keys_with_ragged_key_length(Lq, Lkv, D):
+    """k (and its tangent) expanded along the sequence (stride 0): the rows that a partial last key block pads alias
+    row 0 instead of reading as zeros, so the kernels have to switch those keys off themselves -- in the forward through
+    the scores, in the backward also where dS meets K again for dQ (head dim 72 does it through a spare contraction slot,
+    the others with selects; 256 x 200 and 150 x 130 take the single-pass backward, 300 x 290 the kernel pair).
+    With identical keys dQ = (sum_j dS_ij) k is exactly zero, while a padded key left on would add -delta_i P k = O(0.1)."""
+    B, H, dtype = 2, 2, torch.bfloat16
+    (q, _, v, tq, _, tv, do), (gq, _, gv, gtq, _, gtv, gdo) = _case(B, Lq, H, D, dtype, seed=Lq + Lkv + D, Lkv=Lkv)
+    g = torch.Generator().manual_seed(11)
+    krow, tkrow = (torch.randn(B, 1, H, D, generator=g).to(dtype) for _ in range(2))
+    ex = lambda t: t.float().expand(B, Lkv, H, D).contiguous()
+    gex = lambda t: t.to(DEV).expand(B, Lkv, H, D)
+    scale = D ** -0.5
+    before = _lib.relayout_copies
+    o, to, lse = _lib.fwd_jvp(gq, gex(krow), gv, gtq, gex(tkrow), gtv, scale)[:3]
+    o_ref, to_ref = ao.base_attn_jvp(q, ex(krow), v, tq, ex(tkrow), tv)
+    _check("o", o, o_ref, 2e-2)
+    _check("to", to, to_ref, 2e-2)
+    dq, dk, dv = _lib.bwd(gdo, gq, gex(krow), gv, o, lse, scale)
+    assert _lib.relayout_copies == before
+    dq_ref, dk_ref, dv_ref = ao.base_attn_grads(q, ex(krow), v, do)
+    assert float(dq_ref.abs().max()) <= 1e-4 and float(dq.float().abs().max()) <= 2e-2, float(dq.float().abs().max())
+    _check("dk", dk, dk_ref, 2e-2)
+    _check("dv", dv, dv_ref, 2e-2)
+
+
 # ---- the operator as the model calls it -------------------------------------
 def test_attn_op_hip_under_func_jvp_and_backward():
     B, L, H, D = 2, 256, 4, 64
